@@ -13,6 +13,48 @@ from typing import Optional
 KV_BLOCK_SIZE = 32          # tokens per KV page: one MFMA k-step (16x16x32) of the P·V product
 
 
+@dataclass(frozen=True)
+class MixerSpec:
+    """One layer of a heterogeneous stack (``ModelConfig.layer_specs``): which sequence mixer it has, the mixer's sizes and
+    constants, and its feed-forward.  Fields a mixer kind does not use stay at their defaults.
+
+    ``kind``: ``"attention"`` (grouped-query softmax attention over a sliding window, unit-RMS queries / keys, per-head
+    temperature and logarithmic distance penalty), ``"latent_attention"`` (keys / values expanded from a cached low-rank
+    latent + one shared rotated key part) or ``"lightning"`` (linear attention with a per-head decay and a recurrent state)."""
+    kind: str
+    heads: int
+    dim: int                            # per-head query / key size (latent attention: the unrotated part)
+    vdim: int
+    kv_heads: int = 0                   # attention: key / value heads
+    scale: float = 1.0                  # multiplies q·k
+    window: int = 0                     # attention: a query sees itself and the window-1 tokens before it (0: all)
+    kv_rank: int = 0                    # latent attention: size of the cached latent
+    rot_dim: int = 0                    # latent attention: size of the rotated query / key part
+    rot_base: float = 10000.0
+    rot_dims: int = 0                   # leading entries of the rotated part that are actually rotated
+    decay: tuple = ()                   # lightning: per-head state decay
+    ff: int = 0                         # feed-forward inner width (0: the layer has none)
+    ff_kind: str = "dense"
+
+    @property
+    def stateful(self) -> bool:
+        return self.kind == "lightning"
+
+    @property
+    def cache_row(self) -> tuple:
+        """Widths of the per-token rows this mixer keeps in the paged cache: ``(key row, value row)``; a latent mixer keeps
+        one row (latent | rotated key) that serves as both; a recurrent one keeps none."""
+        if self.kind == "attention":
+            return self.kv_heads * self.dim, self.kv_heads * self.vdim
+        if self.kind == "latent_attention":
+            return self.kv_rank + self.rot_dim, 0
+        return 0, 0
+
+    @property
+    def state_shape(self) -> tuple:
+        return (self.heads, self.dim, self.vdim) if self.kind == "lightning" else ()
+
+
 @dataclass
 class ModelConfig:
     name: str = "llama3-8b"
@@ -36,6 +78,30 @@ class ModelConfig:
     dtype: str = "bfloat16"
     bos_token_id: int = 1
     eos_token_id: int = 2
+    # heterogeneous stacks (arch "rodelix"): one MixerSpec per layer; ``loop = (start, stop, times)`` runs layers
+    # start … stop-1 ``times`` times in a row with the same weights (every pass has its own cache and state, and every pass
+    # but the first starts by adding the embedding output to the stream)
+    layer_specs: tuple = ()
+    loop: Optional[tuple] = None
+    residual_mult: float = 1.0          # a sublayer's normalised output enters the stream times this
+    logit_softcap: float = 0.0          # logits ← cap · tanh(logits / cap); 0: off
+
+    @property
+    def layer_runs(self) -> tuple:
+        """Execution order of a heterogeneous stack: ``(layer index, starts a repeated pass)`` per layer run."""
+        n = len(self.layer_specs)
+        a, b, times = self.loop if self.loop else (0, 0, 1)
+        if b <= a:
+            return tuple((i, False) for i in range(n))
+        runs = [(i, False) for i in range(a)]
+        for p in range(times):
+            runs += [(i, p > 0 and i == a) for i in range(a, b)]
+        return tuple(runs + [(i, False) for i in range(b, n)])
+
+    @property
+    def stateful(self) -> bool:
+        """Sequences carry state besides their cache pages (recurrent mixers, token shift): no prefix sharing, no forks."""
+        return bool(self.layer_specs)
 
     @property
     def q_per_kv(self) -> int:
@@ -43,6 +109,18 @@ class ModelConfig:
 
     def param_count(self) -> int:
         h, i, v, l = self.hidden_size, self.intermediate_size, self.vocab_size, self.num_layers
+        if self.layer_specs:
+            tot = 2 * v * h + 2 * h
+            for m in self.layer_specs:
+                tot += 9 * h + 2 * h * m.ff
+                if m.kind == "attention":
+                    tot += h * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) + m.heads * m.vdim * h
+                elif m.kind == "latent_attention":
+                    tot += h * (m.heads * (m.dim + m.rot_dim) + m.kv_rank + m.rot_dim) + m.kv_rank * m.heads * (m.dim + m.vdim) \
+                        + m.heads * m.vdim * h
+                else:
+                    tot += h * m.heads * (2 * m.dim + 2 * m.vdim) + m.heads * m.vdim * h
+            return tot
         attn = h * (self.num_heads + 2 * self.num_kv_heads) * self.head_dim + self.num_heads * self.head_dim * h
         if self.arch == "opt":
             mlp = 2 * h * i
@@ -50,6 +128,54 @@ class ModelConfig:
             mlp = 3 * h * i * max(self.num_experts, 1)
         emb = v * h * (1 if self.tie_embeddings else 2)
         return l * (attn + mlp) + emb
+
+
+def _rodelix_spec(entry: dict) -> MixerSpec:
+    m, mlp = entry["mixer"], entry.get("mlp")
+    kind = entry["type"]
+    common = dict(kind=kind, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                  ff=int(mlp["ff"]) if mlp else 0, ff_kind=(mlp or {}).get("kind", "dense"))
+    if kind == "attention":
+        return MixerSpec(kv_heads=int(m["kv_heads"]), scale=float(m["scale"]), window=int(m["mask"]["size"]), **common)
+    if kind == "latent_attention":
+        rot = m["rot"]
+        return MixerSpec(scale=float(m["scale"]), kv_rank=int(m["kv_rank"]), rot_dim=int(m["rot_dim"]),
+                         rot_base=float(rot["base"]), rot_dims=int(rot["dims"]), **common)
+    if kind == "lightning":
+        return MixerSpec(decay=tuple(float(d) for d in m["decay"]), **common)
+    raise ValueError(f"unknown mixer type {kind!r}")
+
+
+def rodelix_config(cfg: dict, name: str = "rodelix", dtype: str = "bfloat16") -> ModelConfig:
+    """``ModelConfig`` of a Rodelix checkpoint from the dict its ``config.json`` holds."""
+    specs = tuple(_rodelix_spec(e) for e in cfg["layers"])
+    for s in specs:
+        if s.ff and s.ff_kind != "dense":
+            raise ValueError(f"unknown feed-forward kind {s.ff_kind!r}")
+    loop = cfg.get("loop")
+    first_attn = next((s for s in specs if s.kind != "lightning"), specs[0])
+    return ModelConfig(name=name, arch="rodelix", vocab_size=int(cfg["vocab"]), hidden_size=int(cfg["width"]),
+                       intermediate_size=max(s.ff for s in specs), num_layers=len(specs), num_heads=first_attn.heads,
+                       num_kv_heads=max(first_attn.kv_heads, 1), head_dim=first_attn.dim, max_position=1 << 24,
+                       rms_eps=float(cfg["norm"]["eps"]), dtype=dtype, bos_token_id=0, eos_token_id=-1,
+                       layer_specs=specs, loop=(int(loop["start"]), int(loop["stop"]), int(loop["times"])) if loop else None,
+                       residual_mult=float(cfg.get("residual_mult", 1.0)), logit_softcap=float(cfg.get("logit_softcap") or 0.0))
+
+
+_CONFIG_READERS = {"Rodelix": rodelix_config}
+
+
+def load_model_config(path: str, dtype: Optional[str] = None) -> ModelConfig:
+    """Model configuration of a checkpoint folder: ``config.json``'s ``architecture`` names the reader."""
+    import json
+    import os
+    with open(os.path.join(path, "config.json")) as fh:
+        raw = json.load(fh)
+    arch = raw.get("architecture")
+    if arch not in _CONFIG_READERS:
+        raise ValueError(f"no reader for architecture {arch!r} (have {sorted(_CONFIG_READERS)})")
+    kw = {"dtype": dtype} if dtype else {}
+    return _CONFIG_READERS[arch](raw, name=os.path.basename(os.path.normpath(path)) or arch.lower(), **kw)
 
 
 MODEL_PRESETS: dict[str, ModelConfig] = {
@@ -105,6 +231,21 @@ MODEL_PRESETS: dict[str, ModelConfig] = {
     "tiny-mixtral-8e": ModelConfig(name="tiny-mixtral-8e", arch="mixtral", vocab_size=512, hidden_size=128,
                                    intermediate_size=256, num_layers=2, num_heads=16, num_kv_heads=8, head_dim=8,
                                    max_position=512, num_experts=8, top_k_experts=2, dtype="float32"),
+    # heterogeneous stack: window attention, lightning, latent attention; layers 1-2 run twice
+    "tiny-rodelix": rodelix_config({
+        "vocab": 384, "width": 128, "residual_mult": 0.5, "logit_softcap": 20.0, "norm": {"eps": 1e-5},
+        "loop": {"start": 1, "stop": 3, "times": 2},
+        "layers": [
+            {"type": "attention", "mlp": {"kind": "dense", "ff": 256},
+             "mixer": {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 16, "scale": 0.2, "mask": {"size": 40}}},
+            {"type": "lightning", "mlp": {"kind": "dense", "ff": 256},
+             "mixer": {"heads": 2, "dim": 32, "vdim": 64, "decay": [0.9, 0.98]}},
+            {"type": "latent_attention", "mlp": None,
+             "mixer": {"heads": 4, "dim": 16, "rot_dim": 8, "vdim": 32, "kv_rank": 64, "scale": 0.25,
+                       "rot": {"base": 10000.0, "dims": 8}}},
+            {"type": "attention", "mlp": {"kind": "dense", "ff": 128},
+             "mixer": {"heads": 2, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": 70}}}]},
+        name="tiny-rodelix", dtype="float32"),
     "tiny-opt": ModelConfig(name="tiny-opt", arch="opt", vocab_size=512, hidden_size=64,
                             intermediate_size=128, num_layers=2, num_heads=4, num_kv_heads=4,
                             head_dim=16, max_position=512, pos_offset=2, tie_embeddings=True,

@@ -42,12 +42,23 @@ int build_batch(BlockManager& bm, i64arr seq_ids, i32arr num_computed, i32arr nu
                         query_start_loc.mutable_data());
 }
 
+void fill_state_slots(const BlockManager& bm, i64arr seq_ids, i32out out) {
+  const int B = static_cast<int>(seq_ids.size());
+  if (out.size() < B) throw std::invalid_argument("fill_state_slots: output too small");
+  bm.fill_state_slots(B, seq_ids.data(), out.mutable_data());
+}
+
 }  // namespace
 
 PYBIND11_MODULE(_runtime, m) {
   m.doc() = "dli_amd host runtime: paged-KV block manager and batch builder";
   py::class_<BlockManager>(m, "BlockManager")
-      .def(py::init<int, int, bool>(), py::arg("num_blocks"), py::arg("block_size"), py::arg("prefix_caching") = true)
+      .def(py::init<int, int, bool, int>(), py::arg("num_blocks"), py::arg("block_size"), py::arg("prefix_caching") = true,
+           py::arg("num_state_slots") = 0)
+      .def_property_readonly("num_state_slots", &BlockManager::num_state_slots)
+      .def_property_readonly("num_free_state_slots", &BlockManager::num_free_state_slots)
+      .def("state_slot", &BlockManager::state_slot)
+      .def("fill_state_slots", &fill_state_slots)
       .def_property_readonly("num_blocks", &BlockManager::num_blocks)
       .def_property_readonly("block_size", &BlockManager::block_size)
       .def_property_readonly("num_free", &BlockManager::num_free)

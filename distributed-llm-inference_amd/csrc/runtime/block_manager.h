@@ -37,15 +37,30 @@ struct Seq {
   int hashed_blocks = 0;    // leading blocks whose chain hash has been computed
   uint64_t chain = 0;       // hash of block hashed_blocks-1 (0 at the root)
   bool no_publish = false;  // chain lost (copy-on-write below the hashed prefix): commit() leaves this sequence alone
+  int state_slot = -1;      // row of the per-sequence state tensors (recurrent mixers, token shift); -1: none
 };
 
 class BlockManager {
  public:
-  BlockManager(int num_blocks, int block_size, bool prefix_caching)
-      : bs_(block_size), caching_(prefix_caching), blocks_(num_blocks) {
+  // num_state_slots > 0: models whose sequences carry fixed-size state besides their pages.  Every sequence then owns one
+  // slot from its first allocate() to free_seq(); allocate() fails while none is free.  Such state cannot be rebuilt from
+  // shared pages, so prefix caching must be off and fork() is refused.
+  BlockManager(int num_blocks, int block_size, bool prefix_caching, int num_state_slots = 0)
+      : bs_(block_size), caching_(prefix_caching), blocks_(num_blocks), num_slots_(num_state_slots) {
     if (num_blocks <= 0 || block_size <= 0) throw std::invalid_argument("num_blocks and block_size must be > 0");
+    if (num_state_slots < 0) throw std::invalid_argument("num_state_slots must be >= 0");
+    if (num_state_slots > 0 && prefix_caching) throw std::invalid_argument("state slots and prefix caching exclude each other");
     free_.reserve(num_blocks);
     for (int i = num_blocks - 1; i >= 0; --i) free_.push_back(i);  // pop_back hands out 0,1,2,…
+    for (int i = num_state_slots - 1; i >= 0; --i) free_slots_.push_back(i);
+  }
+
+  int num_state_slots() const { return num_slots_; }
+  int num_free_state_slots() const { return static_cast<int>(free_slots_.size()); }
+  int state_slot(int64_t id) const { return at(id).state_slot; }
+  // state slot of every sequence of a step, in batch order
+  void fill_state_slots(int B, const int64_t* seq_ids, int32_t* out) const {
+    for (int i = 0; i < B; ++i) out[i] = at(seq_ids[i]).state_slot;
   }
 
   int num_blocks() const { return static_cast<int>(blocks_.size()); }
@@ -81,10 +96,17 @@ class BlockManager {
 
   // Grow the block table so that `total_tokens` fit.  All-or-nothing.
   bool allocate(int64_t id, int total_tokens) {
+    auto found = seqs_.find(id);
+    const bool fresh = found == seqs_.end();
+    const int have = fresh ? 0 : static_cast<int>(found->second.blocks.size());
+    const int need = (total_tokens + bs_ - 1) / bs_ - have;
+    const bool want_slot = num_slots_ > 0 && (fresh || found->second.state_slot < 0);
+    if (need > num_free() || (want_slot && free_slots_.empty())) return false;   // nothing taken, no entry left behind
     Seq& s = seqs_[id];
-    const int need = (total_tokens + bs_ - 1) / bs_ - static_cast<int>(s.blocks.size());
-    if (need <= 0) return true;
-    if (need > num_free()) return false;
+    if (want_slot) {
+      s.state_slot = free_slots_.back();
+      free_slots_.pop_back();
+    }
     for (int i = 0; i < need; ++i) s.blocks.push_back(pop_free());
     return true;
   }
@@ -92,6 +114,7 @@ class BlockManager {
   bool can_allocate(int64_t id, int total_tokens) const {
     auto it = seqs_.find(id);
     const int have = it == seqs_.end() ? 0 : static_cast<int>(it->second.blocks.size());
+    if (num_slots_ > 0 && (it == seqs_.end() || it->second.state_slot < 0) && free_slots_.empty()) return false;
     return (total_tokens + bs_ - 1) / bs_ - have <= num_free();
   }
 
@@ -119,12 +142,14 @@ class BlockManager {
     if (it == seqs_.end()) return;
     auto& v = it->second.blocks;
     for (auto r = v.rbegin(); r != v.rend(); ++r) release(*r);  // tail first → tail is evicted first
+    if (it->second.state_slot >= 0) free_slots_.push_back(it->second.state_slot);
     seqs_.erase(it);
   }
 
   // Child shares every block of the parent (n>1 sampling / beam style forks).
   void fork(int64_t parent, int64_t child) {
     const Seq& p = at(parent);
+    if (num_slots_ > 0) throw std::runtime_error("fork: sequences with state slots cannot share pages");
     if (seqs_.count(child)) throw std::runtime_error("fork: child exists");
     Seq c = p;
     for (int b : c.blocks) ++blocks_[b].ref;
@@ -255,6 +280,8 @@ class BlockManager {
   bool caching_;
   std::vector<Block> blocks_;
   std::vector<int> free_;
+  int num_slots_ = 0;
+  std::vector<int> free_slots_;
   std::unordered_map<uint64_t, int> cache_;
   std::unordered_map<int64_t, Seq> seqs_;
   int lru_head_ = -1, lru_tail_ = -1, lru_size_ = 0;

@@ -41,8 +41,13 @@ class LLMEngine:
         self._last_result_time = 0.0
         self.async_scheduling = self._default_async() if cfg.async_scheduling is None else bool(cfg.async_scheduling)
         if self.ctx.is_driver:
-            self.bm = BlockManager(self.runner.num_blocks, KV_BLOCK_SIZE, cfg.cache.enable_prefix_caching)
+            # sequences of a stateful stack (recurrent mixers, token shift) own a state slot next to their pages; what a page
+            # holds cannot stand for the state at its end, so their prefixes are never shared
+            stateful = self.runner.stateful
+            self.bm = BlockManager(self.runner.num_blocks, KV_BLOCK_SIZE, cfg.cache.enable_prefix_caching and not stateful,
+                                   self.runner.num_state_slots)
             self.scheduler = Scheduler(cfg.sched, self.bm)
+            self.scheduler.share_pages = not stateful
             self.scheduler.seq_ids = self._seq_ids
             self.scheduler.max_copies_per_step = ModelRunner.MAX_COW
         else:

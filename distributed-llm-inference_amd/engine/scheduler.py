@@ -56,6 +56,7 @@ class Scheduler:
         self.seq_ids = None                                # iterator of fresh sequence ids (set by the engine)
         self.shed: list[Request] = []                      # finished with status "shed"; the engine reports them
         self.max_copies_per_step = 256                     # copy-on-write pairs one launch takes (ModelRunner.MAX_COW)
+        self.share_pages = True                            # False: sequences carry state that pages do not hold — n > 1 children recompute
         self.num_shed = 0
         # TPOT controller state
         self.dyn_budget = cfg.max_num_batched_tokens        # current total-token target of a step
@@ -357,7 +358,7 @@ class Scheduler:
         import dataclasses
         req.forked = True
         k = req.n_samples - 1
-        room = self.bm.num_free - self.watermark_blocks >= k
+        room = self.share_pages and self.bm.num_free - self.watermark_blocks >= k
         queued = []
         for i in range(1, req.n_samples):
             child = Request(f"{req.req_id}#{i}", next(self.seq_ids), req.tokens[:req.num_prompt],

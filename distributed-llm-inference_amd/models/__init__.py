@@ -15,10 +15,12 @@ import torch
 
 from ..config import ModelConfig
 from ..parallel.state import SINGLE, ParallelContext
+from .layers import random_full_tensor
 from .llama import LlamaForCausalLM
 from .opt import OPTForCausalLM
+from .rodelix import RodelixForCausalLM
 
-_ARCH = {"llama": LlamaForCausalLM, "mixtral": LlamaForCausalLM, "opt": OPTForCausalLM}
+_ARCH = {"llama": LlamaForCausalLM, "mixtral": LlamaForCausalLM, "opt": OPTForCausalLM, "rodelix": RodelixForCausalLM}
 
 
 def torch_dtype(name: str) -> torch.dtype:
@@ -50,6 +52,12 @@ def init_random(model, seed: int = 0) -> None:
             w.init_const(1.0)
         elif kind == "zeros":
             w.init_const(0.0)
+        elif kind == "half":
+            w.init_const(0.5)
+        elif kind == "small":                                # per-head constants of order one (kept positive)
+            w.load_full(random_full_tensor(name, w.full_shape, torch.float32, w.data.device, seed, 1.0).abs() * 0.5)
+        elif w.data.dim() == 2 and hasattr(model, "checkpoint_sources"):
+            w.init_random(name, seed, std=w.full_shape[1] ** -0.5)   # unit-gain projections: the stack has no trained scale
         else:
             w.init_random(name, seed)
 
@@ -94,8 +102,12 @@ class _Shards:
 def load_safetensors(model, path: str) -> None:
     cfg = model.cfg
     shards = _Shards(path)
+    fused = model.checkpoint_sources() if hasattr(model, "checkpoint_sources") else None
     for name, w, _kind in model.named_weights():
-        if ".experts.w" in name:
+        if fused is not None:                                # the model names its checkpoint tensors itself
+            keys = fused.get(name, [name])
+            full = torch.cat([shards.get(k) for k in keys], dim=0) if len(keys) > 1 else shards.get(keys[0])
+        elif ".experts.w" in name:
             full = torch.stack([torch.cat([shards.get(k) for k in ks], dim=0) for ks in _expert_sources(name, cfg)])
         else:
             keys, dim = _hf_sources(name, cfg)

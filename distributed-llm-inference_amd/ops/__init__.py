@@ -17,6 +17,7 @@ import torch
 from . import reference as ref
 from .gemm_plan import PLAN as _PLAN, TAIL as _TAIL
 from .kv_layout import allocate_kv_cache, bytes_per_block, kv_cache_shapes  # noqa: F401
+from . import seqmix  # noqa: F401,E402  (heterogeneous stacks: norms with token shift, token-major attention, linear-attention scan)
 
 _SO = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_C.so")
 _lib = None
@@ -75,6 +76,11 @@ class AttnMetadata:
     prefill_tile_seq: Optional[torch.Tensor] = None
     prefill_tile_q0: Optional[torch.Tensor] = None
     num_prefill_tiles: int = 0
+    # stacks with per-sequence state and token-major caches (ops/seqmix.py): batch row of every token (-1: padding), state
+    # slot of every batch row (-1: none), and the LAUNCHED number of batch rows (the valid count is counts[3])
+    token_seq: Optional[torch.Tensor] = None        # int32 [T]
+    state_slots: Optional[torch.Tensor] = None      # int32 [B]
+    num_seqs: int = 0
 
 
 def prefill_tile_tokens(num_heads: int, num_kv_heads: int) -> int:

@@ -1,0 +1,250 @@
+"""Ops of the heterogeneous decoder stacks (``models/mixers.py``): layer norm with token shift, the
+post-norm residual update, token-major paged attention with a sliding window / distance penalty / two-part
+scores (latent attention), the decayed linear-attention scan over per-sequence state, and the small
+element-wise pieces around them.
+
+Same contract as the rest of ``dli_amd.ops``: GPU tensors go to the gfx950 kernels
+(``csrc/kernels/seqmix.hip``, ``torch.ops.dli.sm_*``), CPU tensors to the fp32 torch references below.  The
+residual stream, norm statistics, scores, softmax weights, rotation angles and the recurrent state are fp32 in
+both; activations between GEMMs are the model dtype (bf16 or fp32).
+
+Cache layout of these mixers: *token-major* pages ``[num_blocks, KV_BLOCK_SIZE, row]`` — one contiguous row per
+token (all key heads, or latent | rotated key), addressed by the same slot ids (``page · 32 + offset``) as the
+other caches.  State tensors are ``[slots, …]`` fp32 rows addressed by ``AttnMetadata.state_slots``.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..config import KV_BLOCK_SIZE
+
+
+def _hip():
+    from . import hip
+    return hip()
+
+
+def _act_ok(x: torch.Tensor) -> bool:
+    if not x.is_cuda:
+        return False
+    if x.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"the sequence-mixer kernels take bfloat16 or float32 activations, got {x.dtype}")
+    return True
+
+
+def _ln(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float) -> torch.Tensor:
+    mu = x.mean(-1, keepdim=True)
+    d = x - mu
+    return d * torch.rsqrt((d * d).mean(-1, keepdim=True) + eps) * w + b
+
+
+def rotary_inv_freq(base: float, dims: int, device="cpu") -> torch.Tensor:
+    """float64 ``[dims/2]``: ``base**(-2i/dims)`` — the kernels multiply by the position in double and reduce the angle
+    before the fp32 sine / cosine, so position 10⁶ is as exact as position 1."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).to(device)
+
+
+# ------------------------------------------------------------------------------------ norms
+def layer_norm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """``(x - mean) / sqrt(var + eps) · w + b`` over fp32 rows; ``out_dtype`` result."""
+    if x.is_cuda:
+        return _hip().sm_layer_norm(x, w, b, eps, out_dtype == torch.bfloat16)
+    return _ln(x.float(), w, b, eps).to(out_dtype)
+
+
+def ln_shift(x: torch.Tensor, add: Optional[torch.Tensor], w: torch.Tensor, b: torch.Tensor, eps: float, mix: torch.Tensor,
+             state: torch.Tensor, meta, out_dtype: torch.dtype):
+    """Pre-norm of a mixer with token shift.  ``x`` fp32 ``[T, W]`` (``add``: added first — the stream's restart term);
+    ``g = layer_norm(x)``; result row ``t`` = ``g[t] + (g[t-1] - g[t]) · mix`` where ``g[t-1]`` is the previous token of the
+    same sequence: the row above inside a chunk, the sequence's ``state`` row at a chunk start, zero at position 0.  The
+    state row becomes ``g`` of the sequence's last token of this step.  Returns ``(h, x)`` with ``x`` the (new) stream."""
+    if x.is_cuda:
+        return _hip().sm_ln_shift(x, add, w, b, eps, mix, state, meta.positions, meta.token_seq, meta.query_start_loc,
+                                  meta.state_slots, meta.counts, meta.num_seqs, out_dtype == torch.bfloat16)
+    if add is not None:
+        x = x + add
+    g = _ln(x, w, b, eps)
+    prev = torch.zeros_like(g)
+    prev[1:] = g[:-1]
+    B = meta.num_decode + meta.num_prefill
+    qsl = meta.query_start_loc[:B + 1].tolist()
+    slots = meta.state_slots[:B].tolist()
+    for i in range(B):
+        t0, t1 = qsl[i], qsl[i + 1]
+        if t1 <= t0 or slots[i] < 0:
+            continue
+        prev[t0] = state[slots[i]] if int(meta.positions[t0]) > 0 else 0.0
+        state[slots[i]] = g[t1 - 1]
+    return (g + (prev - g) * mix).to(out_dtype), x
+
+
+def add_ln(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, mult: float,
+           w2: Optional[torch.Tensor] = None, b2: Optional[torch.Tensor] = None,
+           out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """In place on the fp32 stream: ``x += mult · layer_norm(y; w, b)``; with ``w2`` / ``b2`` also returns
+    ``layer_norm(x; w2, b2)`` (the next sublayer's input) — one pass over the row."""
+    if x.is_cuda:
+        return _hip().sm_add_ln(x, y, w, b, eps, mult, w2, b2, out_dtype == torch.bfloat16)
+    x.add_(_ln(y.float(), w, b, eps), alpha=mult)
+    return None if w2 is None else _ln(x, w2, b2, eps).to(out_dtype)
+
+
+def rms_gate(o: torch.Tensor, w: torch.Tensor, eps: float, gate: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """``o / rms(o) · w · sigmoid(gate)`` per row (``o`` fp32 ``[T, N]``; ``gate`` a row-strided view)."""
+    if o.is_cuda:
+        return _hip().sm_rms_gate(o, w, eps, gate, out_dtype == torch.bfloat16)
+    y = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps) * w
+    return (y * torch.sigmoid(gate.float())).to(out_dtype)
+
+
+def relu2(x: torch.Tensor) -> torch.Tensor:
+    """``max(x, 0)²`` element-wise."""
+    if _act_ok(x):
+        return _hip().sm_relu2(x)
+    z = torch.clamp(x.float(), min=0.0)
+    return (z * z).to(x.dtype)
+
+
+def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """fp32 ``cap · tanh(logits / cap)``."""
+    if logits.is_cuda:
+        return _hip().sm_softcap(logits, cap)
+    return cap * torch.tanh(logits.float() / cap)
+
+
+# ------------------------------------------------------------------------------------ cache writers
+def qk_norm_cache(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor, eps: float, slot_mapping: torch.Tensor,
+                  k_cache: torch.Tensor, v_cache: torch.Tensor, H: int, G: int, D: int, Dv: int) -> None:
+    """``qkv [T, H·D + G·D + G·Dv]``: every query and key head is divided by its root mean square and multiplied by
+    ``qw`` / ``kw`` (fp32 ``[D]``); queries are written back in place, keys and values go to the token-major cache rows
+    ``slot_mapping`` (< 0: skipped)."""
+    if _act_ok(qkv):
+        _hip().sm_qk_norm_cache(qkv, qw, kw, eps, slot_mapping, k_cache, v_cache, H, G, D, Dv)
+        return
+    T = qkv.shape[0]
+    q = qkv[:, :H * D].float().view(T, H, D)
+    k = qkv[:, H * D:(H + G) * D].float().view(T, G, D)
+    q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps) * qw
+    k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps) * kw
+    qkv[:, :H * D] = q.reshape(T, H * D).to(qkv.dtype)
+    keep = slot_mapping >= 0
+    s = slot_mapping[keep].long()
+    k_cache.view(-1, G * D)[s] = k.reshape(T, G * D)[keep].to(k_cache.dtype)
+    v_cache.view(-1, G * Dv)[s] = qkv[:, (H + G) * D:][keep].to(v_cache.dtype)
+
+
+def _rotate(v: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, dims: int) -> torch.Tensor:
+    """v fp32 ``[T, …, R]``: pairs (2i, 2i+1) of the first ``dims`` entries turned by ``position · inv_freq[i]``."""
+    ang = positions.double()[:, None] * inv_freq[None, :]
+    cos, sin = ang.cos().float(), ang.sin().float()
+    while cos.dim() < v.dim():
+        cos, sin = cos.unsqueeze(1), sin.unsqueeze(1)
+    a, b = v[..., 0:dims:2], v[..., 1:dims:2]
+    out = v.clone()
+    out[..., 0:dims:2] = a * cos - b * sin
+    out[..., 1:dims:2] = b * cos + a * sin
+    return out
+
+
+def latent_prep(q: torch.Tensor, dkv: torch.Tensor, cw: torch.Tensor, eps: float, positions: torch.Tensor,
+                inv_freq: torch.Tensor, rot_dims: int, slot_mapping: torch.Tensor, cache: torch.Tensor,
+                H: int, D: int, R: int, C: int) -> None:
+    """Latent attention, per token: the first ``C`` entries of ``dkv [T, C+R]`` divided by their root mean square times
+    ``cw`` are the latent, the last ``R`` the shared key part, rotated for the token's position; both go to the cache row
+    ``[latent | rotated key]``.  The rotated part (last ``R`` of every ``D+R`` head slice) of ``q`` is rotated in place."""
+    if _act_ok(q):
+        _hip().sm_latent_prep(q, dkv, cw, eps, positions, inv_freq, rot_dims, slot_mapping, cache, H, D, R, C)
+        return
+    T = q.shape[0]
+    c = dkv[:, :C].float()
+    c = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps) * cw
+    kr = _rotate(dkv[:, C:].float(), positions, inv_freq, rot_dims)
+    qv = q.unflatten(1, (H, D + R))
+    qv[:, :, D:] = _rotate(qv[:, :, D:].float(), positions, inv_freq, rot_dims).to(q.dtype)
+    keep = slot_mapping >= 0
+    s = slot_mapping[keep].long()
+    cache.view(-1, C + R)[s] = torch.cat([c, kr], dim=-1)[keep].to(cache.dtype)
+
+
+# ------------------------------------------------------------------------------------ attention over token-major pages
+def token_attention(out: torch.Tensor, q1: torch.Tensor, q2: Optional[torch.Tensor], k_cache: torch.Tensor,
+                    v_cache: Optional[torch.Tensor], meta, G: int, Dv: int, scale: float, window: int = 0,
+                    temp: Optional[torch.Tensor] = None, r1: Optional[torch.Tensor] = None,
+                    r2: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Softmax attention of this step's tokens over their sequences' cached rows (which already hold this step's keys).
+
+    ``q1 [T, H, D1]`` (and ``q2 [T, H, D2]``) against key rows ``[G, D1 + D2]``: ``score = (q1·k[:D1] + q2·k[D1:]) · scale ·
+    temp[h] − r1[h] · ln(1 + r2[h] · distance)``; query head ``h`` reads key / value head ``h // (H/G)``.  ``v_cache`` None:
+    the values are the first ``Dv`` entries of the key rows (latent attention: the cached latent is key and value).
+    ``window`` > 0: a query at position ``p`` sees positions ``p-window+1 … p``; 0: all up to ``p``.  Views may be strided
+    (last dim contiguous).  Writes ``out [T, H, Dv]``."""
+    if _act_ok(q1):
+        _hip().sm_token_attention(out, q1, q2, k_cache, v_cache, meta.block_tables, meta.positions, meta.token_seq,
+                                  G, Dv, scale, window, temp, r1, r2)
+        return out
+    T, H, D1 = q1.shape
+    rowk = k_cache.shape[-1]
+    D2 = 0 if q2 is None else q2.shape[2]
+    Dk = D1 + D2
+    assert rowk == G * Dk
+    B = meta.num_decode + meta.num_prefill
+    qsl = meta.query_start_loc[:B + 1].tolist()
+    kflat = k_cache.view(-1, rowk)
+    vflat = kflat if v_cache is None else v_cache.view(-1, v_cache.shape[-1])
+    for i in range(B):
+        t0, t1 = qsl[i], qsl[i + 1]
+        if t1 <= t0:
+            continue
+        pos = meta.positions[t0:t1].long()
+        L = int(pos[-1]) + 1
+        lo = max(int(pos[0]) - window + 1, 0) if window > 0 else 0
+        j = torch.arange(lo, L)
+        slots = meta.block_tables[i, j // KV_BLOCK_SIZE].long() * KV_BLOCK_SIZE + j % KV_BLOCK_SIZE
+        K = kflat[slots].float().view(-1, G, Dk)
+        V = (vflat[slots].float().view(-1, G, vflat.shape[-1] // G))[..., :Dv]
+        q = q1[t0:t1].float() if q2 is None else torch.cat([q1[t0:t1].float(), q2[t0:t1].float()], dim=-1)
+        rep = H // G
+        Kh, Vh = K.repeat_interleave(rep, dim=1), V.repeat_interleave(rep, dim=1)      # [L', H, ·]
+        s = torch.einsum("nhd,lhd->nhl", q, Kh) * scale
+        if temp is not None:
+            s = s * temp.view(1, H, 1)
+        dist = (pos[:, None] - j[None, :])                                             # [n, L']
+        if r1 is not None:
+            s = s - r1.view(1, H, 1) * torch.log1p(r2.view(1, H, 1) * dist.clamp(min=0).float().unsqueeze(1))
+        hidden = dist < 0
+        if window > 0:
+            hidden = hidden | (dist >= window)
+        s = s.masked_fill(hidden.unsqueeze(1), float("-inf"))
+        out[t0:t1] = torch.einsum("nhl,lhd->nhd", torch.softmax(s, dim=-1), Vh).to(out.dtype)
+    return out
+
+
+# ------------------------------------------------------------------------------------ decayed linear attention
+def lightning_scan(qkvg: torch.Tensor, state: torch.Tensor, meta, H: int, D: int, Dv: int, decay: torch.Tensor) -> torch.Tensor:
+    """``qkvg [T, 2·H·D + 2·H·Dv]`` = ``[q | k | v | gate]`` (pre-activation; the gate columns are not read).  Per sequence
+    and head, token by token: ``S ← decay[h] · S + silu(k) silu(v)ᵀ``, ``o = Sᵀ silu(q)`` with ``S`` = the sequence's fp32
+    ``state[slot, h]`` ``[D, Dv]`` (zero at position 0), written back after the step's last token.  Returns fp32 ``[T, H·Dv]``."""
+    if _act_ok(qkvg):
+        return _hip().sm_lightning_scan(qkvg, state, meta.positions, meta.query_start_loc, meta.state_slots, meta.counts,
+                                        meta.num_seqs, H, D, Dv, decay)
+    T = qkvg.shape[0]
+    act = torch.nn.functional.silu(qkvg[:, :2 * H * D + H * Dv].float())
+    q, k, v = act[:, :H * D].view(T, H, D), act[:, H * D:2 * H * D].view(T, H, D), act[:, 2 * H * D:].view(T, H, Dv)
+    o = torch.zeros(T, H, Dv)
+    B = meta.num_decode + meta.num_prefill
+    qsl = meta.query_start_loc[:B + 1].tolist()
+    slots = meta.state_slots[:B].tolist()
+    lam = decay.view(H, 1, 1)
+    for i in range(B):
+        t0, t1 = qsl[i], qsl[i + 1]
+        if t1 <= t0 or slots[i] < 0:
+            continue
+        S = state[slots[i]].clone() if int(meta.positions[t0]) > 0 else torch.zeros(H, D, Dv)
+        for t in range(t0, t1):
+            S = lam * S + k[t].unsqueeze(2) * v[t].unsqueeze(1)
+            o[t] = torch.einsum("hde,hd->he", S, q[t])
+        state[slots[i]] = S
+    return o.view(T, H * Dv)

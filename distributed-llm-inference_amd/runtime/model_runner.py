@@ -56,8 +56,11 @@ class ModelRunner:
         self.on_gpu = device.type == "cuda"
         mcfg = cfg.model
         self.dtype = torch_dtype(mcfg.dtype)
-        if self.on_gpu and self.dtype != torch.bfloat16:
-            self.dtype = torch.bfloat16                      # the HIP kernels are bf16
+        # stacks with their own cache / state layout (models/mixers.py): token-major pages + per-sequence state rows; their
+        # kernels also exist in fp32
+        self.stateful = mcfg.stateful
+        if self.on_gpu and self.dtype != torch.bfloat16 and not self.stateful:
+            self.dtype = torch.bfloat16                      # the HIP kernels of the paged-KV families are bf16
         t0 = time.perf_counter()
         self.model = build_model(mcfg, self.ctx, device, self.dtype, cfg.seed, cfg.weights_path, cfg.quantization)
         self.load_seconds = time.perf_counter() - t0
@@ -68,8 +71,16 @@ class ModelRunner:
         # every rank sizes from its OWN free memory; only the driver's count feeds the block manager, so the group
         # takes the minimum — a worker with fewer pages than the driver would be handed slots past its cache
         self.num_blocks = self.ctx.all_min_int(self._decide_num_blocks())
-        self.kv_caches = allocate_kv_cache(mcfg.num_layers, self.num_blocks, self.local_kv_heads, mcfg.head_dim,
-                                           self.kv_dtype, device)
+        # one state slot per sequence a step can hold (+ the sequences whose last token is still in flight keep theirs)
+        self.num_state_slots = cfg.sched.max_num_seqs if self.stateful else 0
+        if self.stateful:
+            if cfg.cache.kv_dtype == "fp8" or cfg.quantization:
+                raise ValueError("fp8 caches / W8A8 are not implemented for stacks with token-major caches")
+            self.kv_dtype = self.dtype
+            self.kv_caches = self.model.allocate_caches(self.num_blocks, self.num_state_slots, device)
+        else:
+            self.kv_caches = allocate_kv_cache(mcfg.num_layers, self.num_blocks, self.local_kv_heads, mcfg.head_dim,
+                                               self.kv_dtype, device)
         self._alloc_buffers()
         if self.ctx.distributed and self.on_gpu and cfg.use_hip_graphs:
             import torch.distributed as dist
@@ -89,7 +100,8 @@ class ModelRunner:
     def _decide_num_blocks(self) -> int:
         c = self.cfg
         m = c.model
-        per_block = bytes_per_block(m.num_layers, self.local_kv_heads, m.head_dim, self.kv_dtype)
+        per_block = (self.model.bytes_per_block() if self.stateful else
+                     bytes_per_block(m.num_layers, self.local_kv_heads, m.head_dim, self.kv_dtype))
         if c.cache.num_blocks is not None:
             return int(c.cache.num_blocks)
         if not self.on_gpu:
@@ -140,6 +152,7 @@ class ModelRunner:
                   ("top_k", B), ("temp", B), ("top_p", B), ("seeds", 2 * B), ("steps", 2 * B),
                   ("src", B), ("tile_seq", max_tiles), ("tile_q0", max_tiles), ("cow", 2 * self.MAX_COW),
                   ("counts", 4), ("dwork", 4 * self.items_cap), ("dred", 4 * B),
+                  ("tok_seq", T if self.stateful else 0), ("state_slot", B if self.stateful else 0),
                   ("bt", B * self.max_blocks_per_seq)]
         self.layout, off = {}, 0
         for name, n in fields:
@@ -224,8 +237,11 @@ class ModelRunner:
             n_tiles = len(ts)
             nv["tile_seq"][:n_tiles] = ts
             nv["tile_q0"][:n_tiles] = t0
-        n_items, n_reds, n_parts = self._stage_decode_work(nd, cap_items)
-        nv["counts"][:4] = (n_items, n_reds, n_tiles, 0)
+        n_items, n_reds, n_parts = (0, 0, 0) if self.stateful else self._stage_decode_work(nd, cap_items)
+        if self.stateful:                                    # batch row of every token, state slot of every batch row
+            nv["tok_seq"][:T] = np.repeat(np.arange(B, dtype=np.int32), batch.num_new)
+            bm.fill_state_slots(seq_ids, nv["state_slot"])
+        nv["counts"][:4] = (n_items, n_reds, n_tiles, B)
         return B, T, S, n_tiles, n_src, n_items, n_reds, n_parts
 
     def _stage_decode_work(self, nd: int, cap_items: int = 0):
@@ -253,7 +269,9 @@ class ModelRunner:
                             counts=dv["counts"], decode_items=n_items, decode_reds=n_reds, decode_max_parts=self.items_cap,
                             counts_on_device=counts_on_device,
                             prefill_tile_seq=dv["tile_seq"], prefill_tile_q0=dv["tile_q0"],
-                            num_prefill_tiles=n_tiles)
+                            num_prefill_tiles=n_tiles,
+                            token_seq=dv["tok_seq"][:T] if self.stateful else None,
+                            state_slots=dv["state_slot"] if self.stateful else None, num_seqs=B)
 
     # ------------------------------------------------------------------ forward + sample
     def _sample_rows(self, h_rows, S):
@@ -364,6 +382,27 @@ class ModelRunner:
 
     def execute(self, batch, bm) -> np.ndarray:
         return self.collect(self.launch(batch, bm))
+
+    @torch.inference_mode()
+    def forward_logits(self, batch, bm, token_rows) -> torch.Tensor:
+        """One scheduled step with logits instead of samples (trace replay, tooling): the batch is staged, copied in and run
+        through the model exactly as ``launch`` does — same step buffer, same kernels, same cache and state updates — then
+        the LM head is applied to the flattened token rows ``token_rows``.  Returns fp32 ``[len(token_rows), vocab]`` on the
+        host (empty without rows; the step has completed either way).  Single-process engines only."""
+        assert not self.ctx.distributed, "forward_logits drives one rank"
+        self._bind_host(self._host_idx ^ 1)
+        B, T, _S, n_tiles, _n_src, n_items, n_reds, _ = self._stage(batch, bm)
+        self._copy_in()
+        if _DEBUG_BOUNDS:
+            self._check_bounds(B, T, 0)
+        h = self.model(self.dv["input"][:T], self._meta(B, T, batch.num_decode, n_items, n_reds, n_tiles), self.kv_caches)
+        self.stats["eager_steps"] += 1
+        if len(token_rows) == 0:
+            if self.on_gpu:
+                torch.cuda.synchronize()
+            return torch.empty(0, self.cfg.model.vocab_size)
+        rows = torch.as_tensor(np.asarray(token_rows, dtype=np.int64)).to(self.device)
+        return self.model.compute_logits(h.index_select(0, rows)).float().cpu()
 
     HEADER_FIELDS = 12
 
@@ -566,6 +605,9 @@ class ModelRunner:
             self.n_qsl[B + 1:bucket + 1] = np.arange(B + 1, bucket + 1)
             nv["last"][B:bucket] = np.arange(B, bucket)
             nv["src"][B:bucket] = -1
+            if self.stateful:
+                nv["tok_seq"][B:bucket] = -1
+                nv["state_slot"][B:bucket] = -1
             self._pad_sampler_rows(B, bucket)
 
     def _pad_mixed(self, T: int, S: int, tb: int, sb: int):
@@ -575,6 +617,8 @@ class ModelRunner:
             self.n_slot[T:tb] = -1
             self.n_pos[T:tb] = 0
             self.n_input[T:tb] = 0
+            if self.stateful:
+                self.nv["tok_seq"][T:tb] = -1
         rows = self._mixed_caps(tb)[0]
         self.nv["last"][S:max(rows, sb)] = 0
         self._pad_sampler_rows(S, sb)
