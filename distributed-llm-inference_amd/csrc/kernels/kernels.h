@@ -65,6 +65,33 @@ void dense_gemm256_tail_plan(int M, int K, int N_out, bool swiglu, int* tail_til
 void launch_moe_sum(const void* y, bool y_fp32, int n_slabs, int64_t slab_elems, const int* ids, int expert_offset, int E_local,
                     int top_k, int T, int H, void* out, hipStream_t stream);
 
+// heterogeneous decoder stacks (seqmix.hip): fp32 stream / statistics / state, activations bf16 or fp32 (the *_bf16 flags)
+void launch_sm_layer_norm(const float* x, const float* w, const float* b, float eps, int rows, int W, void* out, bool out_bf16,
+                          hipStream_t stream);
+void launch_sm_ln_shift(const float* x, const float* add, float* xout, const float* w, const float* b, const float* mix,
+                        float* state, const int* positions, const int* token_seq, const int* qsl, const int* state_slots,
+                        const int* counts, int rows, int seqs, float eps, int W, void* out, bool out_bf16, hipStream_t stream);
+void launch_sm_add_ln(float* x, const void* y, bool y_bf16, int64_t y_stride, const float* w1, const float* b1, float mult,
+                      const float* w2, const float* b2, float eps, int rows, int W, void* out, bool out_bf16, hipStream_t stream);
+void launch_sm_rms_gate(const float* o, const float* w, float eps, const void* gate, bool gate_bf16, int64_t gate_stride, int rows,
+                        int N, void* out, bool out_bf16, hipStream_t stream);
+void launch_sm_relu2(const void* x, void* out, int64_t n, bool bf16, hipStream_t stream);
+void launch_sm_softcap(const void* x, bool bf16, float* out, float cap, int64_t n, hipStream_t stream);
+void launch_sm_qk_norm_cache(void* qkv, bool bf16, int64_t row_stride, const float* qw, const float* kw, float eps,
+                             const int* slot_mapping, void* k_cache, void* v_cache, int rows, int H, int G, int D, int Dv,
+                             hipStream_t stream);
+void launch_sm_latent_prep(void* q, bool bf16, int64_t q_stride, const void* dkv, int64_t dkv_stride, const float* cw, float eps,
+                           const int* positions, const double* inv_freq, int rot_dims, const int* slot_mapping, void* cache,
+                           int rows, int H, int D, int R, int C, hipStream_t stream);
+void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void* q1, int64_t q1_ts, int64_t q1_hs, int D1,
+                               const void* q2, int64_t q2_ts, int64_t q2_hs, int D2, const void* kc, int rowk, const void* vc,
+                               int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* positions,
+                               const int* token_seq, int rows, int H, int G, float scale, int window, const float* temp,
+                               const float* r1, const float* r2, bool bf16, hipStream_t stream);
+void launch_sm_lightning_scan(const void* qkvg, bool bf16, int64_t row_stride, float* state, const int* positions, const int* qsl,
+                              const int* state_slots, const int* counts, int seqs, int H, int D, int Dv, const float* decay,
+                              float* out, hipStream_t stream);
+
 // custom all-reduce over IPC-mapped peer buffers (custom_all_reduce.hip)
 void* ar_alloc(size_t bytes, bool uncached);
 void ar_free(void* p);

@@ -573,9 +573,28 @@ void ar_all_gather(int64_t st, const Tensor& inp, Tensor out) {
   TORCH_CHECK(rc == 0, "custom all-gather: message of ", inp.numel() * 2, " bytes not supported");
 }
 
+#include "seqmix_bindings.h"
+
 }  // namespace
 
 TORCH_LIBRARY(dli, m) {
+  m.def("sm_layer_norm(Tensor x, Tensor w, Tensor b, float eps, bool out_bf16) -> Tensor", &sm_layer_norm);
+  m.def("sm_ln_shift(Tensor x, Tensor? add, Tensor w, Tensor b, float eps, Tensor mix, Tensor(a!) state, Tensor positions, "
+        "Tensor token_seq, Tensor qsl, Tensor state_slots, Tensor counts, int num_seqs, bool out_bf16) -> (Tensor, Tensor)", &sm_ln_shift);
+  m.def("sm_add_ln(Tensor(a!) x, Tensor y, Tensor w, Tensor b, float eps, float mult, Tensor? w2, Tensor? b2, bool out_bf16) -> Tensor",
+        &sm_add_ln);
+  m.def("sm_rms_gate(Tensor o, Tensor w, float eps, Tensor gate, bool out_bf16) -> Tensor", &sm_rms_gate);
+  m.def("sm_relu2(Tensor x) -> Tensor", &sm_relu2);
+  m.def("sm_softcap(Tensor x, float cap) -> Tensor", &sm_softcap);
+  m.def("sm_qk_norm_cache(Tensor(a!) qkv, Tensor qw, Tensor kw, float eps, Tensor slot_mapping, Tensor(b!) k_cache, Tensor(c!) v_cache, "
+        "int H, int G, int D, int Dv) -> ()", &sm_qk_norm_cache);
+  m.def("sm_latent_prep(Tensor(a!) q, Tensor dkv, Tensor cw, float eps, Tensor positions, Tensor inv_freq, int rot_dims, "
+        "Tensor slot_mapping, Tensor(b!) cache, int H, int D, int R, int C) -> ()", &sm_latent_prep);
+  m.def("sm_token_attention(Tensor(a!) out, Tensor q1, Tensor? q2, Tensor k_cache, Tensor? v_cache, Tensor block_tables, "
+        "Tensor positions, Tensor token_seq, int G, int Dv, float scale, int window, Tensor? temp, Tensor? r1, Tensor? r2) -> ()",
+        &sm_token_attention);
+  m.def("sm_lightning_scan(Tensor qkvg, Tensor(a!) state, Tensor positions, Tensor qsl, Tensor state_slots, Tensor counts, "
+        "int num_seqs, int H, int D, int Dv, Tensor decay) -> Tensor", &sm_lightning_scan);
   m.def("fused_moe(Tensor x, Tensor router_logits, Tensor w13, Tensor w2, int top_k, int expert_offset, int tile_rows=0, Tensor? out=None) -> Tensor",
         &fused_moe);
   m.def("ar_alloc(int bytes, bool uncached) -> int", &ar_alloc);

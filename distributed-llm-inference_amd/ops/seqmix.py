@@ -87,7 +87,8 @@ def add_ln(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, b: torch.Tensor, e
     """In place on the fp32 stream: ``x += mult · layer_norm(y; w, b)``; with ``w2`` / ``b2`` also returns
     ``layer_norm(x; w2, b2)`` (the next sublayer's input) — one pass over the row."""
     if x.is_cuda:
-        return _hip().sm_add_ln(x, y, w, b, eps, mult, w2, b2, out_dtype == torch.bfloat16)
+        h = _hip().sm_add_ln(x, y, w, b, eps, mult, w2, b2, out_dtype == torch.bfloat16)
+        return None if w2 is None else h
     x.add_(_ln(y.float(), w, b, eps), alpha=mult)
     return None if w2 is None else _ln(x, w2, b2, eps).to(out_dtype)
 
