@@ -253,6 +253,17 @@ MODEL_PRESETS: dict[str, ModelConfig] = {
 }
 
 
+def resolve_model(name_or_path: str, dtype: Optional[str] = None, **overrides):
+    """What ``--model`` names: a preset, or a checkpoint folder holding ``config.json`` (then also the default weights path).
+    Returns ``(ModelConfig, weights path or None)``."""
+    import os
+    if os.path.isdir(name_or_path) and os.path.exists(os.path.join(name_or_path, "config.json")):
+        return dataclasses.replace(load_model_config(name_or_path, dtype), **overrides), name_or_path
+    if dtype:
+        overrides["dtype"] = dtype
+    return get_model_config(name_or_path, **overrides), None
+
+
 def get_model_config(name: str, **overrides) -> ModelConfig:
     if name not in MODEL_PRESETS:
         raise KeyError(f"unknown model preset {name!r}; have {sorted(MODEL_PRESETS)}")

@@ -814,8 +814,13 @@ class ModelRunner:
         nv["top_k"][:rows] = 0
         nv["seeds"][:rows] = 1
         nv["steps"][:rows] = 0
-        n_items, n_reds, _ = self._stage_decode_work(B, cap_items)
-        nv["counts"][:4] = (n_items, n_reds, n_tiles, 0)
+        n_items, n_reds, _ = (0, 0, 0) if self.stateful else self._stage_decode_work(B, cap_items)
+        if self.stateful:                                    # row r of the batch uses state slot r (nobody is being served yet)
+            assert rows <= self.num_state_slots, "synthetic batch larger than the state slots"
+            nv["tok_seq"][:B] = i
+            nv["tok_seq"][B:T] = B
+            nv["state_slot"][:rows] = np.arange(rows)
+        nv["counts"][:4] = (n_items, n_reds, n_tiles, rows)
         return rows, T, rows, n_tiles, n_items, n_reds
 
     def _vote(self, ok: bool) -> bool:

@@ -31,7 +31,7 @@ from datetime import datetime, timezone
 
 from aiohttp import web
 
-from ..config import (CacheConfig, EngineConfig, ParallelConfig, SamplingParams, SchedulerConfig, get_model_config)
+from ..config import (CacheConfig, EngineConfig, ParallelConfig, SamplingParams, SchedulerConfig, get_model_config, resolve_model)
 from ..engine.async_engine import AsyncEngine
 from ..engine.tokenizer import get_tokenizer
 
@@ -466,8 +466,11 @@ def engine_config_from_args(a) -> EngineConfig:
         overrides["max_position"] = a.max_position
     if getattr(a, "num_layers", None):
         overrides["num_layers"] = a.num_layers
+    model, found_weights = resolve_model(a.model, getattr(a, "dtype", None), **overrides)
+    if found_weights and not a.weights:
+        a.weights = found_weights                            # a checkpoint folder brings its own weights
     return EngineConfig(
-        model=get_model_config(a.model, **overrides),
+        model=model,
         cache=CacheConfig(kv_dtype=a.kv_dtype, num_blocks=a.num_kv_blocks, gpu_memory_utilization=a.gpu_memory_utilization,
                           enable_prefix_caching=not a.no_prefix_caching,
                           calibration_file=getattr(a, "kv_calibration_file", None)),
@@ -481,7 +484,9 @@ def engine_config_from_args(a) -> EngineConfig:
 
 
 def add_engine_args(ap: argparse.ArgumentParser):
-    ap.add_argument("--model", default="llama3-8b")
+    ap.add_argument("--model", default="llama3-8b", help="a preset name, or a checkpoint folder with config.json + *.safetensors")
+    ap.add_argument("--dtype", default=None, choices=["bfloat16", "float32"],
+                    help="compute dtype (default: the model's; float32 on a GPU only for model families with fp32 kernels)")
     ap.add_argument("--weights", default=None, help="safetensors file/dir (default: random init)")
     ap.add_argument("--tokenizer", default=None, help="HF tokenizer.json (default: byte-level)")
     ap.add_argument("--device", default="auto", choices=["auto", "cuda", "cpu"])
