@@ -823,6 +823,18 @@ class ModelRunner:
         nv["counts"][:4] = (n_items, n_reds, n_tiles, rows)
         return rows, T, rows, n_tiles, n_items, n_reds
 
+    def _save_state_rows(self, n: int) -> list:
+        """Copies of the first ``n`` state slots of every layer run (stateful stacks; a step run twice must start from the
+        same recurrent / token-shift state both times — cache pages, in contrast, are rewritten with the same values)."""
+        if not self.stateful:
+            return []
+        return [(t, t[:n].clone()) for c in self.kv_caches for t in (c.state, c.shift) if t is not None]
+
+    @staticmethod
+    def _restore_state_rows(saved: list) -> None:
+        for t, rows in saved:
+            t[:rows.shape[0]].copy_(rows)
+
     def _vote(self, ok: bool) -> bool:
         return bool(self.ctx.all_min_int(1 if ok else 0))
 
@@ -850,8 +862,10 @@ class ModelRunner:
                 b = min([x for x in decode_keys if x >= 8] or decode_keys)
                 rows, T, S, n_tiles, n_items, n_reds = self._stage_synthetic_decode(b, cap_items=self._decode_caps(b)[0])
                 self._copy_in()
+                saved = self._save_state_rows(rows)
                 le = self._forward_sample(b, b, self._meta(b, b, b, n_items, n_reds, 0)).float().clone()
                 ids_e = self.d_sampled[:b].clone()
+                self._restore_state_rows(saved)              # both runs start from the same per-sequence state
                 self.graphs[b][0].replay()
                 ok, res["graph_vs_eager"] = self._compare_logits(le, self.graphs[b][2].float(), ids_e, self.d_sampled[:b],
                                                                  {"bucket": b})
@@ -879,8 +893,10 @@ class ModelRunner:
                 self._copy_in()
                 # eager over the SAME padded token rows (the GEMMs pick their kernels by row count: 45 rows and 64 rows
                 # differ by bf16 rounding noise, which is not what this test is about), exact launch extents
+                saved = self._save_state_rows(rows)
                 le = self._forward_sample(tb, S, self._meta(rows, tb, nd, n_items, n_reds, n_tiles)).float().clone()
                 ids_e = self.d_sampled[:S].clone()
+                self._restore_state_rows(saved)
                 if ("h", sb) not in self.graphs:
                     self.capture_head_graph(sb)
                 self.graphs[("m", tb)][0].replay()

@@ -177,13 +177,15 @@ def case_generate(tmp, device, dtype, graphs=False):
     from dli_amd.engine.engine import LLMEngine
     W = write_checkpoint(tmp, FULL, 19, bf16=dtype == "bfloat16")
     mcfg, wpath = resolve_model(str(tmp), dtype)
-    eng = LLMEngine(EngineConfig(model=mcfg, weights_path=wpath, device=device, cache=CacheConfig(num_blocks=24),
-                                 sched=SchedulerConfig(max_num_seqs=3, max_num_batched_tokens=48, max_model_len=256,
+    # with graphs: room for the start-up self-test's synthetic mixed step (5 decode rows + a 40-token prompt)
+    seqs, lens = (8, (5, 61, 30, 90, 2, 17, 33, 64, 1, 45, 8)) if graphs else (3, (5, 61, 30, 90, 2))
+    eng = LLMEngine(EngineConfig(model=mcfg, weights_path=wpath, device=device, cache=CacheConfig(num_blocks=8 * seqs),
+                                 sched=SchedulerConfig(max_num_seqs=seqs, max_num_batched_tokens=64, max_model_len=256,
                                                        long_prefill_chunk=40, token_alignment=0),
-                                 use_hip_graphs=graphs, graph_batch_sizes=(1, 2, 4), tune_gemms=False))
+                                 use_hip_graphs=graphs, graph_batch_sizes=(1, 2, 4, 8), tune_gemms=False))
     if graphs:
         eng.warmup()
-    prompts = [tokens(n, FULL["vocab"], 40 + n) for n in (5, 61, 30, 90, 2)]       # five requests, three slots: two wait
+    prompts = [tokens(n, FULL["vocab"], 40 + n) for n in lens]                     # more requests than slots: some wait
     n_new = 12
     outs = eng.generate(None, SamplingParams(temperature=0.0, max_tokens=n_new, ignore_eos=True), prompt_ids=prompts)
     for p, o in zip(prompts, outs):
@@ -195,7 +197,7 @@ def case_generate(tmp, device, dtype, graphs=False):
             if float(top2[0] - top2[1]) > (1e-3 if dtype == "float32" else 0.3):   # skip near-ties
                 assert int(torch.argmax(logits)) == tok
             seq.append(tok)
-    assert eng.bm.num_free == eng.bm.num_blocks and eng.bm.num_free_state_slots == 3
+    assert eng.bm.num_free == eng.bm.num_blocks and eng.bm.num_free_state_slots == seqs
     if graphs:
         assert eng.runner.stats["graph_steps"] > 0, eng.runner.selftest
     return eng
