@@ -8,6 +8,7 @@
     python -m torch.distributed.run --nnodes=1 --nproc-per-node 8 --master-addr 127.0.0.1 --master-port P \
         bench.py --gpus 8 --steps K --warmup W        # the driver's launch: ranks already exist
     python bench.py --sweep                           # SLO frontier: largest offered QPS with ≥ 90 % attainment
+    python bench.py --mixers [--sizes small ...]      # side benchmark: Rodelix stacks beside Llama at equal layer sizes
 
 One rank per GPU.  ``--tp`` consecutive ranks form one tensor-parallel replica (``dp = gpus / tp`` replicas);
 every replica serves its share (round-robin, the router's stateless policy) of ONE global BurstGPT-like trace
@@ -250,6 +251,11 @@ def sustained(done, t_end, seconds, slo):
 
 
 def main():
+    if "--mixers" in sys.argv[1:]:
+        # side benchmark, not the headline: Rodelix stacks beside a Llama stack of equal layer sizes, prefill and decode
+        # throughput through the same engine (benchmarks/bench_mixers.py; its own options follow --mixers)
+        from benchmarks import bench_mixers
+        sys.exit(bench_mixers.main([x for x in sys.argv[1:] if x != "--mixers"]))
     args = parse()
     # ---- stage 0: no GPU touched yet.  Without a torchrun environment, start the ranks ourselves.
     from dli_amd.runtime import launch

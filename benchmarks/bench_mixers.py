@@ -1,0 +1,134 @@
+"""Prefill and decode throughput of Rodelix stacks at layer sizes of a real model, beside a Llama stack of equal
+size (same width, heads, head size and parameter count per layer), both with random weights, both through the same
+engine: requests are added to ``LLMEngine`` and stepped by its scheduler; prefill is timed with one-token requests
+(prompt tokens / wall time), decoding from the step in which the last request got its first token to the end.
+
+    python bench.py --mixers                     # all sizes, one JSON line per (size, model)
+    python benchmarks/bench_mixers.py --sizes small --prompt 1024 --batch 32
+
+Sizes: ``small`` = width 2048, 16 heads of 128, 4 KV heads, FFN 8192 (Llama) — ``large`` = width 4096, 32 heads of 128,
+8 KV heads, FFN 14336 (a Llama-3-8B layer).  The Rodelix stack has one layer per mixer (window attention of 1024 tokens,
+lightning, latent attention with a 512-wide latent + 64 rotated) and a squared-ReLU FFN of 1.5× the Llama FFN width (two
+matrices instead of three: equal parameters); ``rodelix-<mixer>`` rows repeat ONE mixer in every layer so that the three
+can be told apart.  Vocabulary 32000 for all.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+SIZES = {"small": dict(width=2048, heads=16, kv=4, ffn=8192), "large": dict(width=4096, heads=32, kv=8, ffn=14336)}
+LAYERS = 3
+
+
+def rodelix_raw(width, heads, kv, ffn, mixers):
+    ff = {"kind": "dense", "ff": ffn * 3 // 2}
+    mk = {
+        "attention": {"type": "attention", "mlp": ff, "mixer": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128,
+                                                                  "scale": 128 ** -0.5, "mask": {"size": 1024}}},
+        "lightning": {"type": "lightning", "mlp": ff, "mixer": {"heads": heads, "dim": 128, "vdim": 128,
+                                                                  "decay": [1.0 - 2.0 ** -(3 + 5 * h / heads) for h in range(heads)]}},
+        "latent_attention": {"type": "latent_attention", "mlp": ff,
+                             "mixer": {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512,
+                                       "scale": 192 ** -0.5, "rot": {"base": 10000.0, "dims": 64}}},
+    }
+    return {"architecture": "Rodelix", "vocab": 32000, "width": width, "residual_mult": 0.5, "logit_softcap": 30.0,
+            "norm": {"eps": 1e-5}, "layers": [mk[m] for m in mixers]}
+
+
+def model_configs(size):
+    from dli_amd.config import ModelConfig, rodelix_config
+    s = SIZES[size]
+    out = {"llama": ModelConfig(name=f"llama-{size}", arch="llama", vocab_size=32000, hidden_size=s["width"],
+                                intermediate_size=s["ffn"], num_layers=LAYERS, num_heads=s["heads"], num_kv_heads=s["kv"],
+                                head_dim=128, max_position=16384)}
+    kinds = ("attention", "lightning", "latent_attention")
+    out["rodelix"] = rodelix_config(rodelix_raw(s["width"], s["heads"], s["kv"], s["ffn"], kinds), name=f"rodelix-{size}")
+    for k in kinds:
+        out[f"rodelix-{k}"] = rodelix_config(rodelix_raw(s["width"], s["heads"], s["kv"], s["ffn"], (k,) * LAYERS),
+                                             name=f"rodelix-{k}-{size}")
+    return out
+
+
+def run_one(mcfg, prompt, batch, new_tokens, device="cuda", graphs=True):
+    import numpy as np
+    import torch
+    from dli_amd.config import CacheConfig, EngineConfig, SamplingParams, SchedulerConfig
+    from dli_amd.engine.engine import LLMEngine
+    T = 4096
+    pages = batch * ((prompt + new_tokens + 64) // 32 + 1) + 64
+    eng = LLMEngine(EngineConfig(model=mcfg, device=device, cache=CacheConfig(num_blocks=pages, enable_prefix_caching=False),
+                                 sched=SchedulerConfig(max_num_seqs=batch, max_num_batched_tokens=T, max_model_len=prompt + new_tokens + 8,
+                                                       long_prefill_chunk=2048),
+                                 use_hip_graphs=graphs, graph_batch_sizes=(batch,), mixed_step_graphs=False, tune_gemms=False))
+    if graphs:
+        eng.warmup()
+    rng = np.random.default_rng(0)
+
+    def prompts(n):
+        return [rng.integers(3, mcfg.vocab_size, size=prompt).tolist() for _ in range(n)]
+
+    def sync():
+        if device == "cuda":
+            torch.cuda.synchronize()
+
+    eng.generate(None, SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True), prompt_ids=prompts(2))   # warm the eager path
+    # ---- prefill: one-token requests
+    sync()
+    t0 = time.perf_counter()
+    eng.generate(None, SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True), prompt_ids=prompts(batch))
+    sync()
+    t_prefill = time.perf_counter() - t0
+    # ---- decode: from "every request has its first token" to the end
+    ps = prompts(batch)
+    for i, p in enumerate(ps):
+        eng.add_request(f"d{i}", None, SamplingParams(temperature=0.0, max_tokens=new_tokens + 1, ignore_eos=True), p)
+    reqs = [eng.requests[f"d{i}"] for i in range(batch)]
+    while min(r.num_output - r.pending for r in reqs) < 1:
+        eng.step()
+    sync()
+    done0 = sum(r.num_output for r in reqs)
+    t0 = time.perf_counter()
+    steps = 0
+    while eng.has_unfinished():
+        eng.step()
+        steps += 1
+    sync()
+    t_decode = time.perf_counter() - t0
+    made = sum(r.num_output for r in reqs) - done0
+    return {"model": mcfg.name, "params_per_layer_M": round((mcfg.param_count() - 2 * mcfg.vocab_size * mcfg.hidden_size) / LAYERS / 1e6, 1),
+            "prompt": prompt, "batch": batch, "prefill_tokens_per_s": round(batch * prompt / t_prefill),
+            "prefill_ms": round(t_prefill * 1e3, 2), "decode_tokens_per_s": round(made / t_decode),
+            "decode_ms_per_step": round(t_decode / max(steps, 1) * 1e3, 3), "decode_steps": steps,
+            "graph_steps": eng.runner.stats["graph_steps"], "dtype": mcfg.dtype}
+
+
+def main(argv=None, out=None):
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--sizes", default="small,large")
+    ap.add_argument("--models", default="llama,rodelix,rodelix-attention,rodelix-lightning,rodelix-latent_attention")
+    ap.add_argument("--prompt", type=int, default=2048)
+    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--new-tokens", type=int, default=64)
+    ap.add_argument("--device", default="cuda")
+    ap.add_argument("--no-graphs", action="store_true")
+    a = ap.parse_args(argv)
+    out = out or sys.stdout
+    for size in a.sizes.split(","):
+        cfgs = model_configs(size)
+        for name in a.models.split(","):
+            rec = run_one(cfgs[name], a.prompt, a.batch, a.new_tokens, a.device, not a.no_graphs)
+            rec["size"] = size
+            print(json.dumps(rec), file=out, flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

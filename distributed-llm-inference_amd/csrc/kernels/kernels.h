@@ -88,9 +88,15 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
                                int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* positions,
                                const int* token_seq, int rows, int H, int G, float scale, int window, const float* temp,
                                const float* r1, const float* r2, bool bf16, hipStream_t stream);
+bool launch_sm_tile_attention(void* out, int64_t o_ts, int64_t o_hs, const void* q1, int64_t q1_ts, int64_t q1_hs, int D1,
+                              const void* q2, int64_t q2_ts, int64_t q2_hs, int D2, const void* kc, int rowk, const void* vc,
+                              int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* seq_lens,
+                              const int* qsl, const int* tile_seq, const int* tile_q0, int num_tiles, const int* counts, int H,
+                              int G, float scale, int window, const float* temp, const float* r1, const float* r2,
+                              hipStream_t stream);
 void launch_sm_lightning_scan(const void* qkvg, bool bf16, int64_t row_stride, float* state, const int* positions, const int* qsl,
                               const int* state_slots, const int* counts, int seqs, int H, int D, int Dv, const float* decay,
-                              float* out, hipStream_t stream);
+                              float* out, const int* tile_seq, const int* tile_q0, int num_tiles, float* ws, hipStream_t stream);
 
 // custom all-reduce over IPC-mapped peer buffers (custom_all_reduce.hip)
 void* ar_alloc(size_t bytes, bool uncached);

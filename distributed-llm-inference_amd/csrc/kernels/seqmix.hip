@@ -30,6 +30,34 @@ template <> __device__ __forceinline__ void stf<uint16_t>(uint16_t* p, float v) 
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.f + expf(-x)); }
 
+// q (fp32, LDS) · one cache row: 16-byte loads where the row allows them
+template <typename A> __device__ __forceinline__ float dot_row(const float* __restrict__ qs, const A* __restrict__ kr, int n);
+template <> __device__ __forceinline__ float dot_row<float>(const float* __restrict__ qs, const float* __restrict__ kr, int n) {
+  float d = 0.f;
+  int i = 0;
+  if ((n & 3) == 0 && (reinterpret_cast<uintptr_t>(kr) & 15) == 0) {
+    for (; i < n; i += 4) {
+      const f32x4 k = *reinterpret_cast<const f32x4*>(kr + i);
+      d += qs[i] * k[0] + qs[i + 1] * k[1] + qs[i + 2] * k[2] + qs[i + 3] * k[3];
+    }
+  }
+  for (; i < n; ++i) d += qs[i] * kr[i];
+  return d;
+}
+template <> __device__ __forceinline__ float dot_row<uint16_t>(const float* __restrict__ qs, const uint16_t* __restrict__ kr, int n) {
+  float d = 0.f;
+  int i = 0;
+  if ((n & 7) == 0 && (reinterpret_cast<uintptr_t>(kr) & 15) == 0) {
+    for (; i < n; i += 8) {
+      const bf16x8 k = *reinterpret_cast<const bf16x8*>(kr + i);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) d += qs[i + j] * bf2f((uint16_t)k[j]);
+    }
+  }
+  for (; i < n; ++i) d += qs[i] * bf2f(kr[i]);
+  return d;
+}
+
 // mean and 1/sqrt(var + eps) of a row held in LDS (two passes: the variance is the mean squared deviation)
 __device__ __forceinline__ void row_stats(const float* row, int W, float eps, float* red, float& mean, float& inv) {
   float s = 0.f;
@@ -310,8 +338,7 @@ __global__ __launch_bounds__(NT) void token_attention_kernel(
     if (valid) {
       slot = bt[j / kBlockTokens] * kBlockTokens + (j % kBlockTokens);
       const A* kr = kc + (int64_t)slot * rowk + g * Dk;
-      float d = 0.f;
-      for (int i = 0; i < Dk; ++i) d += qs[i] * ldf<A>(kr + i);
+      const float d = dot_row<A>(qs, kr, Dk);
       s = pen ? d - r1h * log1pf(r2h * (float)(p - j)) : d;
     }
     const float mn = fmaxf(m, wave_max(s));
@@ -361,21 +388,199 @@ __global__ __launch_bounds__(NT) void token_attention_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------------------ attention, prefill tiles
+// bf16 only.  One workgroup per (64-query tile of one sequence's chunk, query head); a wave owns 16 queries.  Per 32-key
+// page: the page's key rows (this head's slice) and its value rows, transposed, are staged in LDS once for the four
+// waves; Sᵀ = K·Qᵀ on v_mfma_f32_16x16x32_bf16 (K rows and the register-resident Q rows are both contiguous 16-byte
+// fragments of token-major rows), scale / temperature / distance penalty / window and causal masks and the online
+// softmax in fp32 on the accumulators, then Oᵀ += Vᵀ·Pᵀ with the fp32 weights split into a bf16 head and a bf16
+// remainder (two MFMAs: P enters the product with 16 mantissa bits, not 8).  The lane's eight Sᵀ values (two 16-key
+// tiles) are, in register order, the B fragment of the P·V k-step when the staged V columns sit in the slot order
+// slot(t) = ((t & 15) >> 2)·8 + (t >> 4)·4 + (t & 3).  KSMAX / MTMAX: compile-time bounds of ceil(Dk / 32) and Dv / 16.
+template <int KSMAX, int MTMAX>
+__global__ __launch_bounds__(NT) void tile_attention_kernel(
+    uint16_t* __restrict__ out, int64_t o_ts, int64_t o_hs, const uint16_t* __restrict__ q1, int64_t q1_ts, int64_t q1_hs, int D1,
+    const uint16_t* __restrict__ q2, int64_t q2_ts, int64_t q2_hs, int D2, const uint16_t* __restrict__ kc, int rowk,
+    const uint16_t* __restrict__ vc, int rowv, int vhead, int Dv, const int* __restrict__ block_tables, int max_blocks,
+    const int* __restrict__ seq_lens, const int* __restrict__ qsl, const int* __restrict__ tile_seq,
+    const int* __restrict__ tile_q0, int num_tiles, const int* __restrict__ counts, int H, int G, float scale, int window,
+    const float* __restrict__ temp, const float* __restrict__ r1, const float* __restrict__ r2) {
+  extern __shared__ __align__(16) uint16_t tl[];
+  const int ntiles = counts != nullptr ? min(counts[2], num_tiles) : num_tiles;
+  // the host walks causal tiles longest-first from the END of the list
+  const int tile = num_tiles - 1 - (int)blockIdx.x;
+  if (tile >= ntiles) return;
+  const int h = blockIdx.y;
+  const int seq = tile_seq[tile], q0 = tile_q0[tile];
+  const int t_begin = qsl[seq];
+  const int n_chunk = qsl[seq + 1] - t_begin;
+  const int p0 = seq_lens[seq] - n_chunk;                 // position of the chunk's first token
+  const int nq = min(64, n_chunk - q0);
+  if (nq <= 0) return;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63, g4 = lane >> 4, c = lane & 15;
+  const int Dk = D1 + D2;
+  const int KS = (Dk + 31) >> 5, MT = Dv >> 4;
+  const int KST = KS * 32 + 8;                            // LDS row strides (elements): +16 bytes against bank conflicts
+  constexpr int VST = 40;
+  uint16_t* Ks = tl;
+  uint16_t* Vt = tl + 32 * KST;
+  const int g = h / (H / G);
+
+  // zero the K padding columns once (Dk not a multiple of 32): they are never staged over
+  for (int i = threadIdx.x; i < 32 * (KS * 32 - Dk); i += NT) {
+    const int row = i / (KS * 32 - Dk), col = Dk + i % (KS * 32 - Dk);
+    Ks[row * KST + col] = 0;
+  }
+
+  // this lane's query row as B fragments (zero past Dk and for rows past the tile)
+  const int qi = 16 * wave + c;
+  const bool qvalid = qi < nq;
+  const int64_t tq = t_begin + q0 + qi;
+  bf16x8 qf[KSMAX];
+#pragma unroll
+  for (int s = 0; s < KSMAX; ++s) {
+    const int d = 32 * s + 8 * g4;
+    bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (s < KS && qvalid && d < Dk)
+      v = d < D1 ? *reinterpret_cast<const bf16x8*>(q1 + tq * q1_ts + h * q1_hs + d)
+                 : *reinterpret_cast<const bf16x8*>(q2 + tq * q2_ts + h * q2_hs + (d - D1));
+    qf[s] = v;
+  }
+  const float qmul = scale * (temp != nullptr ? temp[h] : 1.f);
+  const bool pen = r1 != nullptr;
+  const float r1h = pen ? r1[h] : 0.f, r2h = pen ? r2[h] : 0.f;
+  const int pq = p0 + q0 + qi;                            // this lane's query position
+  const int p_first = p0 + q0, p_last = p0 + q0 + nq - 1;
+  const int kb_lo = (window > 0 ? max(p_first - window + 1, 0) : 0) >> 5, kb_hi = p_last >> 5;
+  const int* bt = block_tables + (int64_t)seq * max_blocks;
+
+  float m = -INFINITY, l = 0.f;
+  f32x4 acc[MTMAX];
+#pragma unroll
+  for (int i = 0; i < MTMAX; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int kchunks = Dk >> 3, vchunks = Dv >> 3;
+  for (int kb = kb_lo; kb <= kb_hi; ++kb) {
+    __syncthreads();                                      // everyone is done with the previous page
+    const int64_t page_row = (int64_t)bt[kb] * kBlockTokens;
+    for (int i = threadIdx.x; i < 32 * kchunks; i += NT) {
+      const int row = i / kchunks, ch = i - row * kchunks;
+      *reinterpret_cast<bf16x8*>(Ks + row * KST + 8 * ch) =
+          *reinterpret_cast<const bf16x8*>(kc + (page_row + row) * rowk + g * Dk + 8 * ch);
+    }
+    for (int i = threadIdx.x; i < 32 * vchunks; i += NT) {
+      const int row = i & 31, ch = i >> 5;
+      const bf16x8 v = *reinterpret_cast<const bf16x8*>(vc + (page_row + row) * rowv + g * vhead + 8 * ch);
+      const int slot = ((row & 15) >> 2) * 8 + (row >> 4) * 4 + (row & 3);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) Vt[(8 * ch + j) * VST + slot] = (uint16_t)v[j];
+    }
+    __syncthreads();
+
+    f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < KSMAX; ++s) {
+      if (s < KS) {
+        const bf16x8 ka = *reinterpret_cast<const bf16x8*>(Ks + c * KST + 32 * s + 8 * g4);
+        const bf16x8 kb2 = *reinterpret_cast<const bf16x8*>(Ks + (16 + c) * KST + 32 * s + 8 * g4);
+        sa = mfma16(ka, qf[s], sa);
+        sb = mfma16(kb2, qf[s], sb);
+      }
+    }
+    float sv[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int j = 32 * kb + (r < 4 ? 4 * g4 + r : 16 + 4 * g4 + (r - 4));
+      const bool ok = qvalid && j <= pq && (window <= 0 || j > pq - window);
+      float v = (r < 4 ? sa[r] : sb[r - 4]) * qmul;
+      if (pen) v -= r1h * log1pf(r2h * (float)(pq - j));
+      sv[r] = ok ? v : -INFINITY;
+      mx = fmaxf(mx, sv[r]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mn = fmaxf(m, mx);
+    const float mu = mn == -INFINITY ? 0.f : mn;          // nothing visible yet: keep everything at zero
+    const float corr = expf(m - mu);
+    m = mn;
+    bf16x8 ph, plo;
+    float ps = 0.f;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const float pv = expf(sv[r] - mu);
+      ps += pv;
+      const uint16_t hi = f2bf(pv);
+      ph[r] = (short)hi;
+      plo[r] = (short)f2bf(pv - bf2f(hi));
+    }
+    l = l * corr + ps;
+#pragma unroll
+    for (int i = 0; i < MTMAX; ++i) {
+      if (i < MT) {
+        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vt + (16 * i + c) * VST + 8 * g4);
+        f32x4 a = acc[i];
+        a[0] *= corr; a[1] *= corr; a[2] *= corr; a[3] *= corr;
+        a = mfma16(vf, ph, a);
+        acc[i] = mfma16(vf, plo, a);
+      }
+    }
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!qvalid) return;
+  const float rl = 1.f / l;
+  uint16_t* orow = out + tq * o_ts + h * o_hs;
+#pragma unroll
+  for (int i = 0; i < MTMAX; ++i) {
+    if (i < MT) {
+      bf16x4 o;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[r] = (short)f2bf(acc[i][r] * rl);
+      *reinterpret_cast<bf16x4*>(orow + 16 * i + 4 * g4) = o;
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ linear attention
-// One wave per (sequence, head, 64 value columns): lane e keeps column e of the [D, Dv] state in registers and walks the
-// step's tokens in order: S ← decay·S + silu(k)·silu(v)ᵀ, o = Sᵀ silu(q).  The next token's q / k / v are fetched while
-// the current one is applied.  DMAX: compile-time bound of D (registers per lane).
-template <typename A, int DMAX>
+// S ← decay·S + silu(k)·silu(v)ᵀ, o = Sᵀ silu(q), token by token, with S = a [D, Dv] fp32 state per (sequence, head).
+// One wave per (work item, head, 64 value columns): lane e keeps column e of the state in registers; the next token's
+// q / k / v are fetched while the current one is applied.  DMAX: compile-time bound of D (registers per lane).
+//
+// A work item is either a whole sequence of the step (MODE 0: decode rows — and every sequence when the step has no
+// block list) or one 64-token block of a prefill chunk (the prefill path, three launches so that the blocks of a long
+// chunk run side by side instead of one after the other):
+//   MODE 1  per block: the block's own contribution L = Σ_j decay^(n-1-j) k_j v_jᵀ (state from zero, no output) → ws[block]
+//   prefix  per sequence (lightning_prefix_kernel): walks its blocks in order, leaves in ws[block] the state at the block's
+//           START and in the sequence's state slot the state after its last token: S ← decay^n · S + L
+//   MODE 2  per block: the recurrence again from ws[block], now with outputs.
+// Blocks are the step's prefill tiles (tile_seq / tile_q0, 64 tokens); ws row of a block = (first token >> 6) + batch row
+// (unique: rows of later sequences start at later tokens).
+template <typename A, int DMAX, int MODE>
 __global__ __launch_bounds__(64) void lightning_scan_kernel(const A* __restrict__ qkvg, int64_t row_stride,
                                                             float* __restrict__ state, const int* __restrict__ positions,
                                                             const int* __restrict__ qsl, const int* __restrict__ state_slots,
                                                             const int* __restrict__ counts, int H, int D, int Dv,
-                                                            const float* __restrict__ decay, float* __restrict__ out) {
+                                                            const float* __restrict__ decay, float* __restrict__ out,
+                                                            const int* __restrict__ tile_seq, const int* __restrict__ tile_q0,
+                                                            int num_tiles, float* __restrict__ ws, int single_only) {
   __shared__ float qs[2][DMAX], ks[2][DMAX];
-  const int seq = blockIdx.x;
-  if (seq >= counts[3]) return;
+  int seq, t0, t1;
+  if (MODE == 0) {
+    seq = blockIdx.x;
+    if (seq >= counts[3]) return;
+    t0 = qsl[seq];
+    t1 = qsl[seq + 1];
+    if (single_only && t1 - t0 != 1) return;             // longer chunks take the block path
+  } else {
+    const int tile = blockIdx.x;
+    if (tile >= min(counts[2], num_tiles)) return;
+    seq = tile_seq[tile];
+    t0 = qsl[seq] + tile_q0[tile];
+    t1 = min(t0 + 64, qsl[seq + 1]);
+  }
   const int slot = state_slots[seq];
-  const int t0 = qsl[seq], t1 = qsl[seq + 1];
   if (slot < 0 || t1 <= t0) return;
   const int h = blockIdx.y;
   const int lane = threadIdx.x;
@@ -383,8 +588,9 @@ __global__ __launch_bounds__(64) void lightning_scan_kernel(const A* __restrict_
   const bool active = e < Dv;
   const float lam = decay[h];
   float S[DMAX];
-  float* srow = state + ((int64_t)slot * H + h) * D * Dv;
-  const bool carry = positions[t0] > 0;
+  float* srow = MODE == 0 ? state + ((int64_t)slot * H + h) * D * Dv
+                          : ws + ((int64_t)((t0 >> 6) + seq) * H + h) * D * Dv;
+  const bool carry = MODE == 0 ? positions[t0] > 0 : MODE == 2;
 #pragma unroll
   for (int d = 0; d < DMAX; ++d) S[d] = (carry && active && d < D) ? srow[(int64_t)d * Dv + e] : 0.f;
 
@@ -396,7 +602,7 @@ __global__ __launch_bounds__(64) void lightning_scan_kernel(const A* __restrict_
 #pragma unroll
     for (int r = 0; r < PER; ++r) {
       const int i = lane + 64 * r;
-      nq[r] = i < D ? ldf<A>(row + qoff + i) : 0.f;
+      nq[r] = (MODE != 1 && i < D) ? ldf<A>(row + qoff + i) : 0.f;
       nk[r] = i < D ? ldf<A>(row + koff + i) : 0.f;
     }
     nv = active ? ldf<A>(row + voff + e) : 0.f;
@@ -408,7 +614,7 @@ __global__ __launch_bounds__(64) void lightning_scan_kernel(const A* __restrict_
     for (int r = 0; r < PER; ++r) {
       const int i = lane + 64 * r;
       if (i < DMAX) {
-        qs[buf][i] = silu_f(nq[r]);
+        if (MODE != 1) qs[buf][i] = silu_f(nq[r]);
         ks[buf][i] = silu_f(nk[r]);
       }
     }
@@ -420,15 +626,50 @@ __global__ __launch_bounds__(64) void lightning_scan_kernel(const A* __restrict_
     for (int d = 0; d < DMAX; ++d) {
       if (d < D) {
         S[d] = lam * S[d] + ks[buf][d] * ve;
-        o += S[d] * qs[buf][d];
+        if (MODE != 1) o += S[d] * qs[buf][d];
       }
     }
-    if (active) out[(int64_t)t * H * Dv + (int64_t)h * Dv + e] = o;
+    if (MODE != 1 && active) out[(int64_t)t * H * Dv + (int64_t)h * Dv + e] = o;
   }
-  if (active) {
+  if (MODE != 2 && active) {
 #pragma unroll
     for (int d = 0; d < DMAX; ++d)
       if (d < D) srow[(int64_t)d * Dv + e] = S[d];
+  }
+}
+
+// per (sequence with a chunk of two tokens or more, head, 64 value columns): see above
+__global__ __launch_bounds__(64) void lightning_prefix_kernel(float* __restrict__ state, float* __restrict__ ws,
+                                                              const int* __restrict__ positions, const int* __restrict__ qsl,
+                                                              const int* __restrict__ state_slots, const int* __restrict__ counts,
+                                                              int H, int D, int Dv, const float* __restrict__ decay) {
+  const int seq = blockIdx.x;
+  if (seq >= counts[3]) return;
+  const int t0 = qsl[seq], n = qsl[seq + 1] - t0;
+  const int slot = state_slots[seq];
+  if (slot < 0 || n < 2) return;
+  const int h = blockIdx.y;
+  const int e = blockIdx.z * 64 + threadIdx.x;
+  if (e >= Dv) return;
+  const float lam = decay[h];
+  float lam64 = lam;
+#pragma unroll
+  for (int i = 0; i < 6; ++i) lam64 *= lam64;
+  const int rest = n & 63;
+  float lamr = 1.f;
+  for (int i = 0; i < rest; ++i) lamr *= lam;
+  const bool carry = positions[t0] > 0;
+  const int blocks = (n + 63) >> 6;
+  float* srow = state + ((int64_t)slot * H + h) * D * Dv + e;
+  for (int d = 0; d < D; ++d) {
+    float run = carry ? srow[(int64_t)d * Dv] : 0.f;
+    for (int i = 0; i < blocks; ++i) {
+      float* w = ws + (((int64_t)(((t0 + 64 * i) >> 6) + seq) * H + h) * D + d) * Dv + e;
+      const float own = *w;
+      *w = run;
+      run = ((i == blocks - 1 && rest) ? lamr : lam64) * run + own;
+    }
+    srow[(int64_t)d * Dv] = run;
   }
 }
 
@@ -541,14 +782,62 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
                                                   block_tables, max_blocks, positions, token_seq, H, G, scale, window, temp, r1, r2));
 }
 
+// prefill tiles on the matrix cores (bf16; see tile_attention_kernel).  Returns false when the shapes do not fit its
+// fragments (the caller then runs the per-token kernel over those rows instead).
+bool launch_sm_tile_attention(void* out, int64_t o_ts, int64_t o_hs, const void* q1, int64_t q1_ts, int64_t q1_hs, int D1,
+                              const void* q2, int64_t q2_ts, int64_t q2_hs, int D2, const void* kc, int rowk, const void* vc,
+                              int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* seq_lens,
+                              const int* qsl, const int* tile_seq, const int* tile_q0, int num_tiles, const int* counts, int H,
+                              int G, float scale, int window, const float* temp, const float* r1, const float* r2,
+                              hipStream_t stream) {
+  const int Dk = D1 + D2, KS = (Dk + 31) / 32, MT = Dv / 16;
+  auto al = [](const void* p, int64_t a) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % a == 0; };
+  const bool ok = D1 % 8 == 0 && D2 % 8 == 0 && Dv % 16 == 0 && KS <= 18 && MT <= 32 && rowk % 8 == 0 && rowv % 8 == 0 &&
+                  vhead % 8 == 0 && q1_ts % 8 == 0 && q1_hs % 8 == 0 && q2_ts % 8 == 0 && q2_hs % 8 == 0 && o_ts % 4 == 0 &&
+                  o_hs % 4 == 0 && al(out, 8) && al(q1, 16) && al(q2, 16) && al(kc, 16) && al(vc, 16);
+  if (!ok) return false;
+  if (num_tiles == 0) return true;
+  const size_t lds = (size_t)(32 * (KS * 32 + 8) + Dv * 40) * sizeof(uint16_t);
+  const dim3 grid(num_tiles, H);
+#define SM_TILE(KSM, MTM)                                                                                                        \
+  do {                                                                                                                           \
+    static bool big = false;                                                                                                     \
+    if (lds > 48 * 1024 && !big) {                                                                                               \
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&tile_attention_kernel<KSM, MTM>),                                 \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);                                         \
+      big = true;                                                                                                                \
+    }                                                                                                                            \
+    hipLaunchKernelGGL((tile_attention_kernel<KSM, MTM>), grid, dim3(NT), lds, stream, (uint16_t*)out, o_ts, o_hs,               \
+                       (const uint16_t*)q1, q1_ts, q1_hs, D1, (const uint16_t*)q2, q2_ts, q2_hs, D2, (const uint16_t*)kc, rowk,  \
+                       (const uint16_t*)vc, rowv, vhead, Dv, block_tables, max_blocks, seq_lens, qsl, tile_seq, tile_q0,        \
+                       num_tiles, counts, H, G, scale, window, temp, r1, r2);                                                    \
+  } while (0)
+  if (KS <= 4 && MT <= 8) SM_TILE(4, 8);
+  else if (KS <= 8 && MT <= 16) SM_TILE(8, 16);
+  else SM_TILE(18, 32);
+#undef SM_TILE
+  return true;
+}
+
 void launch_sm_lightning_scan(const void* qkvg, bool bf16, int64_t row_stride, float* state, const int* positions, const int* qsl,
                               const int* state_slots, const int* counts, int seqs, int H, int D, int Dv, const float* decay,
-                              float* out, hipStream_t stream) {
+                              float* out, const int* tile_seq, const int* tile_q0, int num_tiles, float* ws, hipStream_t stream) {
   if (seqs == 0) return;
-  const dim3 grid(seqs, H, (Dv + 63) / 64);
-#define SM_SCAN(DM)                                                                                                                \
-  SM_DISPATCH_BF16(bf16, A, hipLaunchKernelGGL((lightning_scan_kernel<A, DM>), grid, dim3(64), 0, stream, (const A*)qkvg, row_stride, \
-                                               state, positions, qsl, state_slots, counts, H, D, Dv, decay, out))
+  const unsigned zs = (Dv + 63) / 64;
+  const bool blocks = num_tiles > 0 && ws != nullptr;
+#define SM_SCAN(DM)                                                                                                                  \
+  SM_DISPATCH_BF16(bf16, A, {                                                                                                         \
+    hipLaunchKernelGGL((lightning_scan_kernel<A, DM, 0>), dim3(seqs, H, zs), dim3(64), 0, stream, (const A*)qkvg, row_stride, state,  \
+                       positions, qsl, state_slots, counts, H, D, Dv, decay, out, tile_seq, tile_q0, num_tiles, ws, blocks ? 1 : 0);  \
+    if (blocks) {                                                                                                                    \
+      hipLaunchKernelGGL((lightning_scan_kernel<A, DM, 1>), dim3(num_tiles, H, zs), dim3(64), 0, stream, (const A*)qkvg, row_stride,  \
+                         state, positions, qsl, state_slots, counts, H, D, Dv, decay, out, tile_seq, tile_q0, num_tiles, ws, 0);     \
+      hipLaunchKernelGGL(lightning_prefix_kernel, dim3(seqs, H, zs), dim3(64), 0, stream, state, ws, positions, qsl, state_slots,    \
+                         counts, H, D, Dv, decay);                                                                                   \
+      hipLaunchKernelGGL((lightning_scan_kernel<A, DM, 2>), dim3(num_tiles, H, zs), dim3(64), 0, stream, (const A*)qkvg, row_stride,  \
+                         state, positions, qsl, state_slots, counts, H, D, Dv, decay, out, tile_seq, tile_q0, num_tiles, ws, 0);     \
+    }                                                                                                                                \
+  })
   if (D <= 32) SM_SCAN(32);
   else if (D <= 64) SM_SCAN(64);
   else if (D <= 128) SM_SCAN(128);

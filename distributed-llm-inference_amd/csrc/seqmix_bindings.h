@@ -166,9 +166,10 @@ void sm_latent_prep(Tensor q, const Tensor& dkv, const Tensor& cw, double eps, c
 void sm_token_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor>& q2, const Tensor& k_cache,
                         const c10::optional<Tensor>& v_cache, const Tensor& block_tables, const Tensor& positions,
                         const Tensor& token_seq, int64_t G, int64_t Dv, double scale, int64_t window, const c10::optional<Tensor>& temp,
-                        const c10::optional<Tensor>& r1, const c10::optional<Tensor>& r2) {
+                        const c10::optional<Tensor>& r1, const c10::optional<Tensor>& r2, int64_t rows) {
   const bool bf = act_bf16(q1, "q1");
   TORCH_CHECK(q1.dim() == 3 && q1.stride(2) == 1, "q1 must be [T, H, D1] with a contiguous last dim");
+  TORCH_CHECK(rows < 0 || rows <= q1.size(0), "rows past the batch");
   const int64_t T = q1.size(0), H = q1.size(1), D1 = q1.size(2);
   int64_t D2 = 0;
   if (q2.has_value()) {
@@ -202,12 +203,66 @@ void sm_token_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor
                                  q2.has_value() ? q2->data_ptr() : nullptr, q2.has_value() ? q2->stride(0) : 0,
                                  q2.has_value() ? q2->stride(1) : 0, (int)D2, k_cache.data_ptr(), (int)(G * Dk), vc.data_ptr(),
                                  (int)vc.size(2), (int)vhead, (int)Dv, block_tables.data_ptr<int>(), (int)block_tables.size(1),
-                                 positions.data_ptr<int>(), token_seq.data_ptr<int>(), (int)T, (int)H, (int)G, (float)scale, (int)window,
-                                 opt_f32(temp, "temp", H), opt_f32(r1, "r1", H), opt_f32(r2, "r2", H), bf, cur_stream(q1));
+                                 positions.data_ptr<int>(), token_seq.data_ptr<int>(), (int)(rows < 0 ? T : rows), (int)H, (int)G, (float)scale,
+                                 (int)window, opt_f32(temp, "temp", H), opt_f32(r1, "r1", H), opt_f32(r2, "r2", H), bf, cur_stream(q1));
+}
+
+// Prefill tiles (64 queries of one sequence's chunk each) on the matrix cores; bf16 only.  False: shapes the tile kernel does
+// not take — nothing was launched, the caller uses the per-token kernel.
+bool sm_tile_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor>& q2, const Tensor& k_cache,
+                       const c10::optional<Tensor>& v_cache, const Tensor& block_tables, const Tensor& seq_lens, const Tensor& qsl,
+                       const Tensor& tile_seq, const Tensor& tile_q0, int64_t num_tiles, const c10::optional<Tensor>& counts, int64_t G,
+                       int64_t Dv, double scale, int64_t window, const c10::optional<Tensor>& temp, const c10::optional<Tensor>& r1,
+                       const c10::optional<Tensor>& r2) {
+  TORCH_CHECK(q1.is_cuda() && q1.scalar_type() == at::kBFloat16 && q1.dim() == 3 && q1.stride(2) == 1, "q1 must be bfloat16 [T, H, D1]");
+  const int64_t T = q1.size(0), H = q1.size(1), D1 = q1.size(2);
+  int64_t D2 = 0;
+  if (q2.has_value()) {
+    TORCH_CHECK(q2->is_cuda() && q2->scalar_type() == at::kBFloat16 && q2->dim() == 3 && q2->stride(2) == 1 && q2->size(0) == T &&
+                    q2->size(1) == H, "q2 must be [T, H, D2] like q1");
+    D2 = q2->size(2);
+  }
+  TORCH_CHECK(G > 0 && H % G == 0, "query heads must be a multiple of the key heads");
+  const int64_t Dk = D1 + D2;
+  TORCH_CHECK(k_cache.is_cuda() && k_cache.is_contiguous() && k_cache.scalar_type() == at::kBFloat16 && k_cache.dim() == 3 &&
+                  k_cache.size(1) == kSmPageTokens && k_cache.size(2) == G * Dk, "k_cache must be [pages, 32, G*(D1+D2)]");
+  const Tensor& vc = v_cache.has_value() ? *v_cache : k_cache;
+  int64_t vhead = Dk;
+  if (v_cache.has_value()) {
+    TORCH_CHECK(vc.is_cuda() && vc.is_contiguous() && vc.scalar_type() == at::kBFloat16 && vc.dim() == 3 && vc.size(0) == k_cache.size(0) &&
+                    vc.size(1) == kSmPageTokens && vc.size(2) == G * Dv, "v_cache must be [pages, 32, G*Dv]");
+    vhead = Dv;
+  } else {
+    TORCH_CHECK(Dv <= Dk, "values read from the key rows cannot be wider than a key");
+  }
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == at::kBFloat16 && out.dim() == 3 && out.stride(2) == 1 && out.size(0) == T &&
+                  out.size(1) == H && out.size(2) == Dv, "out must be [T, H, Dv]");
+  check_i32(block_tables, "block_tables");
+  check_i32(seq_lens, "seq_lens");
+  check_i32(qsl, "query_start_loc");
+  check_i32(tile_seq, "tile_seq");
+  check_i32(tile_q0, "tile_q0");
+  TORCH_CHECK(block_tables.dim() == 2 && num_tiles >= 0 && tile_seq.numel() >= num_tiles && tile_q0.numel() >= num_tiles,
+              "tile list shorter than the launch");
+  const int* cnt = nullptr;
+  if (counts.has_value()) {
+    check_i32(*counts, "counts");
+    TORCH_CHECK(counts->numel() >= 4, "counts must hold 4 values");
+    cnt = counts->data_ptr<int>();
+  }
+  TORCH_CHECK(r1.has_value() == r2.has_value(), "r1 and r2 come together");
+  return dli::launch_sm_tile_attention(out.data_ptr(), out.stride(0), out.stride(1), q1.data_ptr(), q1.stride(0), q1.stride(1), (int)D1,
+                                       q2.has_value() ? q2->data_ptr() : nullptr, q2.has_value() ? q2->stride(0) : 0,
+                                       q2.has_value() ? q2->stride(1) : 0, (int)D2, k_cache.data_ptr(), (int)(G * Dk), vc.data_ptr(),
+                                       (int)vc.size(2), (int)vhead, (int)Dv, block_tables.data_ptr<int>(), (int)block_tables.size(1),
+                                       seq_lens.data_ptr<int>(), qsl.data_ptr<int>(), tile_seq.data_ptr<int>(), tile_q0.data_ptr<int>(),
+                                       (int)num_tiles, cnt, (int)H, (int)G, (float)scale, (int)window, opt_f32(temp, "temp", H),
+                                       opt_f32(r1, "r1", H), opt_f32(r2, "r2", H), cur_stream(q1));
 }
 
 Tensor sm_lightning_scan(const Tensor& qkvg, Tensor state, const Tensor& positions, const Tensor& qsl, const Tensor& state_slots,
-                         const Tensor& counts, int64_t num_seqs, int64_t H, int64_t D, int64_t Dv, const Tensor& decay) {
+                         const Tensor& counts, int64_t num_seqs, int64_t H, int64_t D, int64_t Dv, const Tensor& decay,
+                         const c10::optional<Tensor>& tile_seq, const c10::optional<Tensor>& tile_q0, int64_t num_tiles) {
   const bool bf = act_bf16(qkvg, "qkvg");
   check_rows(qkvg, "qkvg");
   const int64_t T = qkvg.size(0);
@@ -223,8 +278,22 @@ Tensor sm_lightning_scan(const Tensor& qkvg, Tensor state, const Tensor& positio
   TORCH_CHECK(positions.numel() >= T && counts.numel() >= 4 && num_seqs >= 0 && qsl.numel() >= num_seqs + 1 &&
                   state_slots.numel() >= num_seqs, "step metadata shorter than the batch");
   Tensor out = at::zeros({T, H * Dv}, qkvg.options().dtype(at::kFloat));
+  // block path of prefill chunks: 64-token blocks = the step's prefill tiles; one [H, D, Dv] workspace row per block
+  const int* ts = nullptr;
+  const int* tq = nullptr;
+  Tensor ws;
+  if (num_tiles > 0) {
+    TORCH_CHECK(tile_seq.has_value() && tile_q0.has_value(), "a block list needs tile_seq and tile_q0");
+    check_i32(*tile_seq, "tile_seq");
+    check_i32(*tile_q0, "tile_q0");
+    TORCH_CHECK(tile_seq->numel() >= num_tiles && tile_q0->numel() >= num_tiles, "tile list shorter than the launch");
+    ts = tile_seq->data_ptr<int>();
+    tq = tile_q0->data_ptr<int>();
+    ws = at::empty({T / 64 + num_seqs + 2, H, D, Dv}, state.options());
+  }
   dli::launch_sm_lightning_scan(qkvg.data_ptr(), bf, qkvg.stride(0), state.data_ptr<float>(), positions.data_ptr<int>(),
                                 qsl.data_ptr<int>(), state_slots.data_ptr<int>(), counts.data_ptr<int>(), (int)num_seqs, (int)H, (int)D,
-                                (int)Dv, decay.data_ptr<float>(), out.data_ptr<float>(), cur_stream(qkvg));
+                                (int)Dv, decay.data_ptr<float>(), out.data_ptr<float>(), ts, tq, (int)num_tiles,
+                                num_tiles > 0 ? ws.data_ptr<float>() : nullptr, cur_stream(qkvg));
   return out;
 }

@@ -591,10 +591,14 @@ TORCH_LIBRARY(dli, m) {
   m.def("sm_latent_prep(Tensor(a!) q, Tensor dkv, Tensor cw, float eps, Tensor positions, Tensor inv_freq, int rot_dims, "
         "Tensor slot_mapping, Tensor(b!) cache, int H, int D, int R, int C) -> ()", &sm_latent_prep);
   m.def("sm_token_attention(Tensor(a!) out, Tensor q1, Tensor? q2, Tensor k_cache, Tensor? v_cache, Tensor block_tables, "
-        "Tensor positions, Tensor token_seq, int G, int Dv, float scale, int window, Tensor? temp, Tensor? r1, Tensor? r2) -> ()",
+        "Tensor positions, Tensor token_seq, int G, int Dv, float scale, int window, Tensor? temp, Tensor? r1, Tensor? r2, int rows=-1) -> ()",
         &sm_token_attention);
+  m.def("sm_tile_attention(Tensor(a!) out, Tensor q1, Tensor? q2, Tensor k_cache, Tensor? v_cache, Tensor block_tables, Tensor seq_lens, "
+        "Tensor qsl, Tensor tile_seq, Tensor tile_q0, int num_tiles, Tensor? counts, int G, int Dv, float scale, int window, "
+        "Tensor? temp, Tensor? r1, Tensor? r2) -> bool", &sm_tile_attention);
   m.def("sm_lightning_scan(Tensor qkvg, Tensor(a!) state, Tensor positions, Tensor qsl, Tensor state_slots, Tensor counts, "
-        "int num_seqs, int H, int D, int Dv, Tensor decay) -> Tensor", &sm_lightning_scan);
+        "int num_seqs, int H, int D, int Dv, Tensor decay, Tensor? tile_seq=None, Tensor? tile_q0=None, int num_tiles=0) -> Tensor",
+        &sm_lightning_scan);
   m.def("fused_moe(Tensor x, Tensor router_logits, Tensor w13, Tensor w2, int top_k, int expert_offset, int tile_rows=0, Tensor? out=None) -> Tensor",
         &fused_moe);
   m.def("ar_alloc(int bytes, bool uncached) -> int", &ar_alloc);

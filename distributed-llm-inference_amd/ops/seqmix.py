@@ -14,11 +14,17 @@ other caches.  State tensors are ``[slots, …]`` fp32 rows addressed by ``AttnM
 """
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
 
 from ..config import KV_BLOCK_SIZE
+
+
+TILE_ATTENTION = os.environ.get("DLI_TILE_ATTENTION", "1") != "0"     # A/B knob: prefill tiles on the matrix cores (bf16)
+BLOCK_SCAN = os.environ.get("DLI_BLOCK_SCAN", "1") != "0"             # A/B knob: block-parallel lightning prefill
+PREFILL_TILE_TOKENS = 64                                                # queries per prefill tile of these stacks
 
 
 def _hip():
@@ -183,8 +189,17 @@ def token_attention(out: torch.Tensor, q1: torch.Tensor, q2: Optional[torch.Tens
     ``window`` > 0: a query at position ``p`` sees positions ``p-window+1 … p``; 0: all up to ``p``.  Views may be strided
     (last dim contiguous).  Writes ``out [T, H, Dv]``."""
     if _act_ok(q1):
-        _hip().sm_token_attention(out, q1, q2, k_cache, v_cache, meta.block_tables, meta.positions, meta.token_seq,
-                                  G, Dv, scale, window, temp, r1, r2)
+        lib = _hip()
+        rows = -1
+        if TILE_ATTENTION and q1.dtype == torch.bfloat16 and meta.num_prefill_tiles > 0:
+            # prefill chunks: 64-query tiles on the matrix cores; the per-token kernel keeps the decode rows in front
+            if lib.sm_tile_attention(out, q1, q2, k_cache, v_cache, meta.block_tables, meta.seq_lens, meta.query_start_loc,
+                                     meta.prefill_tile_seq, meta.prefill_tile_q0, meta.num_prefill_tiles,
+                                     meta.counts if meta.counts_on_device else None, G, Dv, scale, window, temp, r1, r2):
+                rows = meta.num_decode
+        if rows != 0:
+            lib.sm_token_attention(out, q1, q2, k_cache, v_cache, meta.block_tables, meta.positions, meta.token_seq,
+                                   G, Dv, scale, window, temp, r1, r2, rows)
         return out
     T, H, D1 = q1.shape
     rowk = k_cache.shape[-1]
@@ -229,8 +244,11 @@ def lightning_scan(qkvg: torch.Tensor, state: torch.Tensor, meta, H: int, D: int
     and head, token by token: ``S ← decay[h] · S + silu(k) silu(v)ᵀ``, ``o = Sᵀ silu(q)`` with ``S`` = the sequence's fp32
     ``state[slot, h]`` ``[D, Dv]`` (zero at position 0), written back after the step's last token.  Returns fp32 ``[T, H·Dv]``."""
     if _act_ok(qkvg):
+        # prefill chunks run block-parallel over the step's 64-token tiles (local states → prefix over blocks → outputs)
+        tiles = meta.num_prefill_tiles if BLOCK_SCAN else 0
         return _hip().sm_lightning_scan(qkvg, state, meta.positions, meta.query_start_loc, meta.state_slots, meta.counts,
-                                        meta.num_seqs, H, D, Dv, decay)
+                                        meta.num_seqs, H, D, Dv, decay, meta.prefill_tile_seq if tiles else None,
+                                        meta.prefill_tile_q0 if tiles else None, tiles)
     T = qkvg.shape[0]
     act = torch.nn.functional.silu(qkvg[:, :2 * H * D + H * Dv].float())
     q, k, v = act[:, :H * D].view(T, H, D), act[:, H * D:2 * H * D].view(T, H, D), act[:, 2 * H * D:].view(T, H, Dv)

@@ -88,7 +88,8 @@ class ModelRunner:
                 cfg.use_hip_graphs = False                   # gloo collectives synchronise the host: not capturable
         self.graphs: dict[int, tuple] = {}
         self.graph_pool = None
-        self.tile_tokens = ops.prefill_tile_tokens(self.local_heads, self.local_kv_heads)
+        self.tile_tokens = (ops.seqmix.PREFILL_TILE_TOKENS if self.stateful else
+                            ops.prefill_tile_tokens(self.local_heads, self.local_kv_heads))
         self.stats = {"graph_steps": 0, "mixed_graph_steps": 0, "eager_steps": 0, "ar_fallbacks": 0}
         self.selftest: dict = {}                             # start-up checks of the fast paths → what got disabled
         self._dumped = False
