@@ -73,8 +73,9 @@ void launch_sm_ln_shift(const float* x, const float* add, float* xout, const flo
                         const int* counts, int rows, int seqs, float eps, int W, void* out, bool out_bf16, hipStream_t stream);
 void launch_sm_add_ln(float* x, const void* y, bool y_bf16, int64_t y_stride, const float* w1, const float* b1, float mult,
                       const float* w2, const float* b2, float eps, int rows, int W, void* out, bool out_bf16, hipStream_t stream);
-void launch_sm_rms_gate(const float* o, const float* w, float eps, const void* gate, bool gate_bf16, int64_t gate_stride, int rows,
-                        int N, void* out, bool out_bf16, hipStream_t stream);
+void launch_sm_rms_gate(const float* o, int parts, const float* w, float eps, const void* gate, bool gate_bf16, int64_t gate_stride,
+                        int rows, int N, void* out, bool out_bf16, hipStream_t stream);
+int sm_lightning_parts(int D);
 void launch_sm_relu2(const void* x, void* out, int64_t n, bool bf16, hipStream_t stream);
 void launch_sm_softcap(const void* x, bool bf16, float* out, float cap, int64_t n, hipStream_t stream);
 void launch_sm_qk_norm_cache(void* qkv, bool bf16, int64_t row_stride, const float* qw, const float* kw, float eps,
@@ -96,7 +97,8 @@ bool launch_sm_tile_attention(void* out, int64_t o_ts, int64_t o_hs, const void*
                               hipStream_t stream);
 void launch_sm_lightning_scan(const void* qkvg, bool bf16, int64_t row_stride, float* state, const int* positions, const int* qsl,
                               const int* state_slots, const int* counts, int seqs, int H, int D, int Dv, const float* decay,
-                              float* out, const int* tile_seq, const int* tile_q0, int num_tiles, float* ws, hipStream_t stream);
+                              float* out, int64_t out_part, const int* tile_seq, const int* tile_q0, int num_tiles, float* ws,
+                              hipStream_t stream);
 
 // custom all-reduce over IPC-mapped peer buffers (custom_all_reduce.hip)
 void* ar_alloc(size_t bytes, bool uncached);

@@ -173,21 +173,25 @@ __global__ __launch_bounds__(NT) void add_ln_kernel(float* __restrict__ x, const
   for (int i = threadIdx.x; i < W; i += NT) stf<O>(out + t * W + i, (sh[i] - mean) * inv * w2[i] + b2[i]);
 }
 
+// o: `parts` planes of partial sums [parts][T][N] (the scan cuts the state rows into parts); the row is their sum
 template <typename G, typename O>
-__global__ __launch_bounds__(NT) void rms_gate_kernel(const float* __restrict__ o, const float* __restrict__ w, float eps,
-                                                      const G* __restrict__ gate, int64_t gate_stride, int N,
-                                                      O* __restrict__ out) {
+__global__ __launch_bounds__(NT) void rms_gate_kernel(const float* __restrict__ o, int parts, int64_t part_stride,
+                                                      const float* __restrict__ w, float eps, const G* __restrict__ gate,
+                                                      int64_t gate_stride, int N, O* __restrict__ out) {
+  extern __shared__ float sh[];
   __shared__ float red[NT / 64];
   const int64_t t = blockIdx.x;
   float s = 0.f;
   for (int i = threadIdx.x; i < N; i += NT) {
-    const float v = o[t * N + i];
+    float v = o[t * N + i];
+    for (int p = 1; p < parts; ++p) v += o[p * part_stride + t * N + i];
+    sh[i] = v;
     s += v * v;
   }
   const float inv = 1.f / sqrtf(block_sum<NT>(s, red) / (float)N + eps);
   for (int i = threadIdx.x; i < N; i += NT) {
     const float g = ldf<G>(gate + t * gate_stride + i);
-    stf<O>(out + t * N + i, o[t * N + i] * inv * w[i] / (1.f + expf(-g)));
+    stf<O>(out + t * N + i, sh[i] * inv * w[i] / (1.f + expf(-g)));
   }
 }
 
@@ -292,99 +296,200 @@ __global__ __launch_bounds__(NT) void latent_prep_kernel(A* __restrict__ q, int6
 }
 
 // ------------------------------------------------------------------------------------------------ attention
-// One workgroup per (token, query head); every wave takes chunks of 64 consecutive keys, a lane per key for the scores
-// (q broadcast from LDS), then lanes over the value columns for P·V (weights and cache rows broadcast by shuffles).
-// Online softmax per wave, the four waves merged through LDS.  Serves decode rows and prefill-chunk tokens alike: a
-// token's position and batch row come from the step metadata, keys from the sequence's block-table row.
-template <typename A, int NV>
+// VPL contiguous elements of a cache row → fp32 (one wide load when the row allows it)
+template <typename A, int VPL>
+__device__ __forceinline__ void load_vals(const A* __restrict__ p, bool wide, float* __restrict__ dst);
+template <int VPL>
+__device__ __forceinline__ void load_vals_f32(const float* __restrict__ p, bool wide, float* __restrict__ dst) {
+  if (wide && VPL >= 4) {
+#pragma unroll
+    for (int i = 0; i < VPL; i += 4) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(p + i);
+      dst[i] = v[0]; dst[i + 1] = v[1]; dst[i + 2] = v[2]; dst[i + 3] = v[3];
+    }
+  } else if (wide && VPL == 2) {
+    const f32x2 v = *reinterpret_cast<const f32x2*>(p);
+    dst[0] = v[0]; dst[1] = v[1];
+  } else {
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) dst[i] = p[i];
+  }
+}
+template <int VPL>
+__device__ __forceinline__ void load_vals_bf16(const uint16_t* __restrict__ p, bool wide, float* __restrict__ dst) {
+  if (wide && VPL == 8) {
+    const bf16x8 v = *reinterpret_cast<const bf16x8*>(p);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dst[i] = bf2f((uint16_t)v[i]);
+  } else if (wide && VPL == 4) {
+    const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[i] = bf2f((uint16_t)v[i]);
+  } else if (wide && VPL == 2) {
+    const uint32_t v = *reinterpret_cast<const uint32_t*>(p);
+    dst[0] = __uint_as_float(v << 16);
+    dst[1] = __uint_as_float(v & 0xffff0000u);
+  } else {
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) dst[i] = bf2f(p[i]);
+  }
+}
+template <> __device__ __forceinline__ void load_vals<float, 1>(const float* p, bool w, float* d) { load_vals_f32<1>(p, w, d); }
+template <> __device__ __forceinline__ void load_vals<float, 2>(const float* p, bool w, float* d) { load_vals_f32<2>(p, w, d); }
+template <> __device__ __forceinline__ void load_vals<float, 4>(const float* p, bool w, float* d) { load_vals_f32<4>(p, w, d); }
+template <> __device__ __forceinline__ void load_vals<float, 8>(const float* p, bool w, float* d) { load_vals_f32<8>(p, w, d); }
+template <> __device__ __forceinline__ void load_vals<uint16_t, 1>(const uint16_t* p, bool w, float* d) { load_vals_bf16<1>(p, w, d); }
+template <> __device__ __forceinline__ void load_vals<uint16_t, 2>(const uint16_t* p, bool w, float* d) { load_vals_bf16<2>(p, w, d); }
+template <> __device__ __forceinline__ void load_vals<uint16_t, 4>(const uint16_t* p, bool w, float* d) { load_vals_bf16<4>(p, w, d); }
+template <> __device__ __forceinline__ void load_vals<uint16_t, 8>(const uint16_t* p, bool w, float* d) { load_vals_bf16<8>(p, w, d); }
+
+// One workgroup per (token, group of HG query heads that read the same key / value head): a key row and a value row are
+// loaded once for the HG heads.  Every wave takes chunks of 64 consecutive keys: a lane per key for the scores (the HG
+// queries broadcast from LDS, the key row in 16-byte pieces), then lanes over the value columns for P·V — lane owns the
+// VPL contiguous columns lane·VPL …, one wide load per key, the key's weight and cache row broadcast as scalars
+// (v_readlane).  Online softmax per wave and head, the four waves merged through LDS.  Serves decode rows and
+// prefill-chunk tokens alike: a token's position and batch row come from the step metadata, keys from the sequence's
+// block-table row.  Value sizes up to 64·VPL.
+template <typename A, int VPL, int HG>
 __global__ __launch_bounds__(NT) void token_attention_kernel(
     A* __restrict__ out, int64_t o_ts, int64_t o_hs, const A* __restrict__ q1, int64_t q1_ts, int64_t q1_hs, int D1,
     const A* __restrict__ q2, int64_t q2_ts, int64_t q2_hs, int D2, const A* __restrict__ kc, int rowk,
     const A* __restrict__ vc, int rowv, int vhead, int Dv, const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ positions, const int* __restrict__ token_seq, int H, int G, float scale, int window,
     const float* __restrict__ temp, const float* __restrict__ r1, const float* __restrict__ r2) {
-  extern __shared__ float sh[];          // q [Dk] | per wave: acc [Dv] | m[4] | l[4]
+  extern __shared__ float sh[];          // q [HG][Dk] | acc [4 waves][HG][Dv] | m [4][HG] | l [4][HG]
+  constexpr int NW = NT / 64;
   const int64_t t = blockIdx.x;
-  const int h = blockIdx.y;
+  const int h0 = blockIdx.y * HG;        // first head of the group (all HG heads share one key / value head)
   const int seq = token_seq[t];
   if (seq < 0) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int Dk = D1 + D2;
   const int p = positions[t];
   const int lo = window > 0 ? max(p - window + 1, 0) : 0;
-  const int g = h / (H / G);
+  const int g = h0 / (H / G);
   float* qs = sh;
-  float* accs = sh + Dk;
-  float* ms = accs + (NT / 64) * Dv;
-  float* ls = ms + NT / 64;
-  const float qmul = scale * (temp != nullptr ? temp[h] : 1.f);
-  for (int i = threadIdx.x; i < Dk; i += NT)
-    qs[i] = qmul * (i < D1 ? ldf<A>(q1 + t * q1_ts + h * q1_hs + i) : ldf<A>(q2 + t * q2_ts + h * q2_hs + (i - D1)));
+  float* accs = sh + HG * Dk;
+  float* ms = accs + NW * HG * Dv;
+  float* ls = ms + NW * HG;
+  for (int i = threadIdx.x; i < HG * Dk; i += NT) {
+    const int hh = i / Dk, d = i - hh * Dk, h = h0 + hh;
+    const float qmul = scale * (temp != nullptr ? temp[h] : 1.f);
+    qs[i] = qmul * (d < D1 ? ldf<A>(q1 + t * q1_ts + h * q1_hs + d) : ldf<A>(q2 + t * q2_ts + h * q2_hs + (d - D1)));
+  }
   __syncthreads();
   const bool pen = r1 != nullptr;
-  const float r1h = pen ? r1[h] : 0.f, r2h = pen ? r2[h] : 0.f;
-  const int* bt = block_tables + (int64_t)seq * max_blocks;
-
-  float m = -INFINITY, l = 0.f;
-  float acc[NV];
+  float r1h[HG], r2h[HG];
 #pragma unroll
-  for (int v = 0; v < NV; ++v) acc[v] = 0.f;
+  for (int hh = 0; hh < HG; ++hh) {
+    r1h[hh] = pen ? r1[h0 + hh] : 0.f;
+    r2h[hh] = pen ? r2[h0 + hh] : 0.f;
+  }
+  const int* bt = block_tables + (int64_t)seq * max_blocks;
+  constexpr int esz = sizeof(A);
+  const bool kwide = (Dk * esz) % 16 == 0 && (rowk * esz) % 16 == 0 && (reinterpret_cast<uintptr_t>(kc) & 15) == 0;
+  const bool vwide = ((int64_t)rowv * esz) % (VPL * esz) == 0 && ((int64_t)vhead * esz) % (VPL * esz) == 0 &&
+                     (reinterpret_cast<uintptr_t>(vc) % (VPL * esz)) == 0 && Dv % VPL == 0;
+  const int e0 = lane * VPL;             // this lane's value columns
 
-  for (int base = lo + wave * 64; base <= p; base += (NT / 64) * 64) {
+  float m[HG], l[HG], acc[HG][VPL];
+#pragma unroll
+  for (int hh = 0; hh < HG; ++hh) {
+    m[hh] = -INFINITY;
+    l[hh] = 0.f;
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) acc[hh][v] = 0.f;
+  }
+
+  for (int base = lo + wave * 64; base <= p; base += NW * 64) {
     const int j = base + lane;
     const bool valid = j <= p;
     int slot = 0;
-    float s = -INFINITY;
+    float s[HG];
+#pragma unroll
+    for (int hh = 0; hh < HG; ++hh) s[hh] = 0.f;
     if (valid) {
       slot = bt[j / kBlockTokens] * kBlockTokens + (j % kBlockTokens);
       const A* kr = kc + (int64_t)slot * rowk + g * Dk;
-      const float d = dot_row<A>(qs, kr, Dk);
-      s = pen ? d - r1h * log1pf(r2h * (float)(p - j)) : d;
+      constexpr int KV = 16 / esz;       // elements per 16-byte piece
+      int i = 0;
+      if (kwide) {
+        for (; i + KV <= Dk; i += KV) {
+          float kv[KV];
+          load_vals<A, KV == 8 ? 8 : 4>(kr + i, true, kv);
+#pragma unroll
+          for (int hh = 0; hh < HG; ++hh) {
+            float d = 0.f;
+#pragma unroll
+            for (int u = 0; u < KV; ++u) d += qs[hh * Dk + i + u] * kv[u];
+            s[hh] += d;
+          }
+        }
+      }
+      for (; i < Dk; ++i) {
+        const float kv = ldf<A>(kr + i);
+#pragma unroll
+        for (int hh = 0; hh < HG; ++hh) s[hh] += qs[hh * Dk + i] * kv;
+      }
     }
-    const float mn = fmaxf(m, wave_max(s));
-    const float corr = expf(m - mn);               // first chunk: exp(-inf) = 0
-    const float pl = valid ? expf(s - mn) : 0.f;
-    l = l * corr + wave_sum(pl);
-    m = mn;
+    float pl[HG];
 #pragma unroll
-    for (int v = 0; v < NV; ++v) acc[v] *= corr;
+    for (int hh = 0; hh < HG; ++hh) {
+      float sv = -INFINITY;
+      if (valid) sv = pen ? s[hh] - r1h[hh] * log1pf(r2h[hh] * (float)(p - j)) : s[hh];
+      const float mn = fmaxf(m[hh], wave_max(sv));
+      const float corr = expf(m[hh] - mn);             // first chunk: exp(-inf) = 0
+      pl[hh] = valid ? expf(sv - mn) : 0.f;
+      l[hh] = l[hh] * corr + wave_sum(pl[hh]);
+      m[hh] = mn;
+#pragma unroll
+      for (int v = 0; v < VPL; ++v) acc[hh][v] *= corr;
+    }
     const int nvalid = min(p - base + 1, 64);
-    for (int jj = 0; jj < nvalid; ++jj) {
-      const float pj = __shfl(pl, jj, 64);
-      const int sj = __shfl(slot, jj, 64);
-      const A* vr = vc + (int64_t)sj * rowv + g * vhead;
+    if (e0 < Dv) {
+      for (int jj = 0; jj < nvalid; ++jj) {
+        const int sj = __builtin_amdgcn_readlane(slot, jj);
+        float vv[VPL];
+        const A* vr = vc + (int64_t)sj * rowv + g * vhead + e0;
+        if (vwide) {
+          load_vals<A, VPL>(vr, true, vv);
+        } else {
 #pragma unroll
-      for (int v = 0; v < NV; ++v) {
-        const int e = lane + 64 * v;
-        if (e < Dv) acc[v] += pj * ldf<A>(vr + e);
+          for (int v = 0; v < VPL; ++v) vv[v] = e0 + v < Dv ? ldf<A>(vr + v) : 0.f;
+        }
+#pragma unroll
+        for (int hh = 0; hh < HG; ++hh) {
+          const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pl[hh]), jj));
+#pragma unroll
+          for (int v = 0; v < VPL; ++v) acc[hh][v] += pj * vv[v];
+        }
       }
     }
   }
 #pragma unroll
-  for (int v = 0; v < NV; ++v) {
-    const int e = lane + 64 * v;
-    if (e < Dv) accs[wave * Dv + e] = acc[v];
-  }
-  if (lane == 0) {
-    ms[wave] = m;
-    ls[wave] = l;
+  for (int hh = 0; hh < HG; ++hh) {
+#pragma unroll
+    for (int v = 0; v < VPL; ++v)
+      if (e0 + v < Dv) accs[(wave * HG + hh) * Dv + e0 + v] = acc[hh][v];
+    if (lane == 0) {
+      ms[wave * HG + hh] = m[hh];
+      ls[wave * HG + hh] = l[hh];
+    }
   }
   __syncthreads();
-  float M = ms[0];
+  for (int i = threadIdx.x; i < HG * Dv; i += NT) {
+    const int hh = i / Dv, e = i - hh * Dv;
+    float M = ms[hh];
 #pragma unroll
-  for (int w = 1; w < NT / 64; ++w) M = fmaxf(M, ms[w]);
-  float L = 0.f;
-  float f[NT / 64];
+    for (int w = 1; w < NW; ++w) M = fmaxf(M, ms[w * HG + hh]);
+    float L = 0.f, o = 0.f;
 #pragma unroll
-  for (int w = 0; w < NT / 64; ++w) {
-    f[w] = expf(ms[w] - M);
-    L += f[w] * ls[w];
-  }
-  for (int e = threadIdx.x; e < Dv; e += NT) {
-    float o = 0.f;
-#pragma unroll
-    for (int w = 0; w < NT / 64; ++w) o += f[w] * accs[w * Dv + e];
-    stf<A>(out + t * o_ts + h * o_hs + e, o / L);
+    for (int w = 0; w < NW; ++w) {
+      const float f = expf(ms[w * HG + hh] - M);
+      L += f * ls[w * HG + hh];
+      o += f * accs[(w * HG + hh) * Dv + e];
+    }
+    stf<A>(out + t * o_ts + (h0 + hh) * o_hs + e, o / L);
   }
 }
 
@@ -564,7 +669,8 @@ __global__ __launch_bounds__(64) void lightning_scan_kernel(const A* __restrict_
                                                             const int* __restrict__ counts, int H, int D, int Dv,
                                                             const float* __restrict__ decay, float* __restrict__ out,
                                                             const int* __restrict__ tile_seq, const int* __restrict__ tile_q0,
-                                                            int num_tiles, float* __restrict__ ws, int single_only) {
+                                                            int num_tiles, float* __restrict__ ws, int single_only, int zs,
+                                                            int DR, int64_t out_part) {
   __shared__ float qs[2][DMAX], ks[2][DMAX];
   int seq, t0, t1;
   if (MODE == 0) {
@@ -584,17 +690,25 @@ __global__ __launch_bounds__(64) void lightning_scan_kernel(const A* __restrict_
   if (slot < 0 || t1 <= t0) return;
   const int h = blockIdx.y;
   const int lane = threadIdx.x;
-  const int e = blockIdx.z * 64 + lane;
+  // blockIdx.z = (part of the D rows, 64-column slice): this wave owns state rows dbase … dbase + DR - 1 (DR ≤ DMAX); the
+  // partial outputs of the parts go to separate planes of `out` and are summed by the consumer (rms_gate_kernel)
+  const int part = blockIdx.z / zs;
+  const int e = (blockIdx.z - part * zs) * 64 + lane;
+  const int dbase = part * DR;
+  const int Dn = min(DR, D - dbase);                   // rows of this part
+  if (Dn <= 0) return;
+  out += part * out_part;
   const bool active = e < Dv;
   const float lam = decay[h];
   float S[DMAX];
-  float* srow = MODE == 0 ? state + ((int64_t)slot * H + h) * D * Dv
-                          : ws + ((int64_t)((t0 >> 6) + seq) * H + h) * D * Dv;
+  float* srow = (MODE == 0 ? state + ((int64_t)slot * H + h) * D * Dv
+                           : ws + ((int64_t)((t0 >> 6) + seq) * H + h) * D * Dv) + (int64_t)dbase * Dv;
   const bool carry = MODE == 0 ? positions[t0] > 0 : MODE == 2;
 #pragma unroll
-  for (int d = 0; d < DMAX; ++d) S[d] = (carry && active && d < D) ? srow[(int64_t)d * Dv + e] : 0.f;
+  for (int d = 0; d < DMAX; ++d) S[d] = (carry && active && d < Dn) ? srow[(int64_t)d * Dv + e] : 0.f;
 
-  const int64_t qoff = (int64_t)h * D, koff = (int64_t)H * D + (int64_t)h * D, voff = 2 * (int64_t)H * D + (int64_t)h * Dv;
+  const int64_t qoff = (int64_t)h * D + dbase, koff = (int64_t)H * D + (int64_t)h * D + dbase,
+                voff = 2 * (int64_t)H * D + (int64_t)h * Dv;
   constexpr int PER = (DMAX + 63) / 64;
   float nq[PER], nk[PER], nv = 0.f;
   auto fetch = [&](int t) {
@@ -602,8 +716,8 @@ __global__ __launch_bounds__(64) void lightning_scan_kernel(const A* __restrict_
 #pragma unroll
     for (int r = 0; r < PER; ++r) {
       const int i = lane + 64 * r;
-      nq[r] = (MODE != 1 && i < D) ? ldf<A>(row + qoff + i) : 0.f;
-      nk[r] = i < D ? ldf<A>(row + koff + i) : 0.f;
+      nq[r] = (MODE != 1 && i < Dn) ? ldf<A>(row + qoff + i) : 0.f;
+      nk[r] = i < Dn ? ldf<A>(row + koff + i) : 0.f;
     }
     nv = active ? ldf<A>(row + voff + e) : 0.f;
   };
@@ -624,7 +738,7 @@ __global__ __launch_bounds__(64) void lightning_scan_kernel(const A* __restrict_
     float o = 0.f;
 #pragma unroll
     for (int d = 0; d < DMAX; ++d) {
-      if (d < D) {
+      if (d < Dn) {
         S[d] = lam * S[d] + ks[buf][d] * ve;
         if (MODE != 1) o += S[d] * qs[buf][d];
       }
@@ -634,7 +748,7 @@ __global__ __launch_bounds__(64) void lightning_scan_kernel(const A* __restrict_
   if (MODE != 2 && active) {
 #pragma unroll
     for (int d = 0; d < DMAX; ++d)
-      if (d < D) srow[(int64_t)d * Dv + e] = S[d];
+      if (d < Dn) srow[(int64_t)d * Dv + e] = S[d];
   }
 }
 
@@ -715,12 +829,13 @@ void launch_sm_add_ln(float* x, const void* y, bool y_bf16, int64_t y_stride, co
                                                                                 y_stride, w1, b1, mult, w2, b2, eps, W, (O*)out)));
 }
 
-void launch_sm_rms_gate(const float* o, const float* w, float eps, const void* gate, bool gate_bf16, int64_t gate_stride, int rows,
-                        int N, void* out, bool out_bf16, hipStream_t stream) {
+void launch_sm_rms_gate(const float* o, int parts, const float* w, float eps, const void* gate, bool gate_bf16, int64_t gate_stride,
+                        int rows, int N, void* out, bool out_bf16, hipStream_t stream) {
   if (rows == 0) return;
-  SM_DISPATCH_BF16(gate_bf16, G, SM_DISPATCH_BF16(out_bf16, O, hipLaunchKernelGGL((rms_gate_kernel<G, O>), dim3(rows), dim3(NT), 0,
-                                                                                   stream, o, w, eps, (const G*)gate, gate_stride,
-                                                                                   N, (O*)out)));
+  const int64_t ps = (int64_t)rows * N;
+  SM_DISPATCH_BF16(gate_bf16, G, SM_DISPATCH_BF16(out_bf16, O, hipLaunchKernelGGL((rms_gate_kernel<G, O>), dim3(rows), dim3(NT),
+                                                                                   N * sizeof(float), stream, o, parts, ps, w, eps,
+                                                                                   (const G*)gate, gate_stride, N, (O*)out)));
 }
 
 void launch_sm_relu2(const void* x, void* out, int64_t n, bool bf16, hipStream_t stream) {
@@ -752,19 +867,19 @@ void launch_sm_latent_prep(void* q, bool bf16, int64_t q_stride, const void* dkv
                                                rot_dims, slot_mapping, (A*)cache, H, D, R, C));
 }
 
-template <typename A>
-static void token_attention_nv(int nv, dim3 grid, size_t lds, hipStream_t stream, A* out, int64_t o_ts, int64_t o_hs, const A* q1,
+template <typename A, int VPL>
+static void token_attention_hg(int hg, dim3 grid, size_t lds, hipStream_t stream, A* out, int64_t o_ts, int64_t o_hs, const A* q1,
                                int64_t q1_ts, int64_t q1_hs, int D1, const A* q2, int64_t q2_ts, int64_t q2_hs, int D2, const A* kc,
                                int rowk, const A* vc, int rowv, int vhead, int Dv, const int* bt, int max_blocks, const int* pos,
                                const int* tseq, int H, int G, float scale, int window, const float* temp, const float* r1,
                                const float* r2) {
-#define SM_ATT(NVV)                                                                                                              \
-  hipLaunchKernelGGL((token_attention_kernel<A, NVV>), grid, dim3(NT), lds, stream, out, o_ts, o_hs, q1, q1_ts, q1_hs, D1, q2,   \
-                     q2_ts, q2_hs, D2, kc, rowk, vc, rowv, vhead, Dv, bt, max_blocks, pos, tseq, H, G, scale, window, temp, r1, r2)
-  if (nv <= 1) SM_ATT(1);
-  else if (nv <= 2) SM_ATT(2);
-  else if (nv <= 4) SM_ATT(4);
-  else SM_ATT(8);
+#define SM_ATT(HGV)                                                                                                              \
+  hipLaunchKernelGGL((token_attention_kernel<A, VPL, HGV>), grid, dim3(NT), lds, stream, out, o_ts, o_hs, q1, q1_ts, q1_hs, D1,  \
+                     q2, q2_ts, q2_hs, D2, kc, rowk, vc, rowv, vhead, Dv, bt, max_blocks, pos, tseq, H, G, scale, window, temp,  \
+                     r1, r2)
+  if (hg == 1) SM_ATT(1);
+  else if (hg == 2) SM_ATT(2);
+  else SM_ATT(4);
 #undef SM_ATT
 }
 
@@ -774,12 +889,24 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
                                const int* token_seq, int rows, int H, int G, float scale, int window, const float* temp,
                                const float* r1, const float* r2, bool bf16, hipStream_t stream) {
   if (rows == 0) return;
-  const size_t lds = (size_t)(D1 + D2 + (NT / 64) * Dv + 2 * (NT / 64)) * sizeof(float);
-  const dim3 grid(rows, H);
+  // heads per workgroup: as many of the heads sharing a key / value head as divide their number and fit the LDS budget
+  const int per = H / G, Dk = D1 + D2;
+  int hg = per % 4 == 0 ? 4 : (per % 2 == 0 ? 2 : 1);
+  auto lds_of = [&](int g) { return (size_t)(g * Dk + (NT / 64) * g * Dv + 2 * (NT / 64) * g) * sizeof(float); };
+  while (hg > 1 && lds_of(hg) > 60 * 1024) hg >>= 1;
+  const size_t lds = lds_of(hg);
+  const dim3 grid(rows, H / hg);
   const int nv = (Dv + 63) / 64;
-  SM_DISPATCH_BF16(bf16, A, token_attention_nv<A>(nv, grid, lds, stream, (A*)out, o_ts, o_hs, (const A*)q1, q1_ts, q1_hs, D1,
-                                                  (const A*)q2, q2_ts, q2_hs, D2, (const A*)kc, rowk, (const A*)vc, rowv, vhead, Dv,
-                                                  block_tables, max_blocks, positions, token_seq, H, G, scale, window, temp, r1, r2));
+#define SM_ATT_V(VPLV)                                                                                                            \
+  SM_DISPATCH_BF16(bf16, A, (token_attention_hg<A, VPLV>(hg, grid, lds, stream, (A*)out, o_ts, o_hs, (const A*)q1, q1_ts, q1_hs, \
+                                                         D1, (const A*)q2, q2_ts, q2_hs, D2, (const A*)kc, rowk, (const A*)vc,   \
+                                                         rowv, vhead, Dv, block_tables, max_blocks, positions, token_seq, H, G,  \
+                                                         scale, window, temp, r1, r2)))
+  if (nv <= 1) SM_ATT_V(1);
+  else if (nv <= 2) SM_ATT_V(2);
+  else if (nv <= 4) SM_ATT_V(4);
+  else SM_ATT_V(8);
+#undef SM_ATT_V
 }
 
 // prefill tiles on the matrix cores (bf16; see tile_attention_kernel).  Returns false when the shapes do not fit its
@@ -819,28 +946,38 @@ bool launch_sm_tile_attention(void* out, int64_t o_ts, int64_t o_hs, const void*
   return true;
 }
 
+// rows of the state one wave keeps: D is cut into parts so that a wave's per-token loop is short and more waves share the work
+int sm_lightning_parts(int D) { return D >= 128 ? 4 : (D >= 64 ? 2 : 1); }
+
 void launch_sm_lightning_scan(const void* qkvg, bool bf16, int64_t row_stride, float* state, const int* positions, const int* qsl,
                               const int* state_slots, const int* counts, int seqs, int H, int D, int Dv, const float* decay,
-                              float* out, const int* tile_seq, const int* tile_q0, int num_tiles, float* ws, hipStream_t stream) {
+                              float* out, int64_t out_part, const int* tile_seq, const int* tile_q0, int num_tiles, float* ws,
+                              hipStream_t stream) {
   if (seqs == 0) return;
-  const unsigned zs = (Dv + 63) / 64;
+  const int zs = (Dv + 63) / 64;
+  const int parts = sm_lightning_parts(D);
+  const int DR = (D + parts - 1) / parts;
+  const unsigned gz = zs * parts;
   const bool blocks = num_tiles > 0 && ws != nullptr;
 #define SM_SCAN(DM)                                                                                                                  \
   SM_DISPATCH_BF16(bf16, A, {                                                                                                         \
-    hipLaunchKernelGGL((lightning_scan_kernel<A, DM, 0>), dim3(seqs, H, zs), dim3(64), 0, stream, (const A*)qkvg, row_stride, state,  \
-                       positions, qsl, state_slots, counts, H, D, Dv, decay, out, tile_seq, tile_q0, num_tiles, ws, blocks ? 1 : 0);  \
+    hipLaunchKernelGGL((lightning_scan_kernel<A, DM, 0>), dim3(seqs, H, gz), dim3(64), 0, stream, (const A*)qkvg, row_stride, state,  \
+                       positions, qsl, state_slots, counts, H, D, Dv, decay, out, tile_seq, tile_q0, num_tiles, ws, blocks ? 1 : 0,  \
+                       zs, DR, out_part);                                                                                            \
     if (blocks) {                                                                                                                    \
-      hipLaunchKernelGGL((lightning_scan_kernel<A, DM, 1>), dim3(num_tiles, H, zs), dim3(64), 0, stream, (const A*)qkvg, row_stride,  \
-                         state, positions, qsl, state_slots, counts, H, D, Dv, decay, out, tile_seq, tile_q0, num_tiles, ws, 0);     \
+      hipLaunchKernelGGL((lightning_scan_kernel<A, DM, 1>), dim3(num_tiles, H, gz), dim3(64), 0, stream, (const A*)qkvg, row_stride,  \
+                         state, positions, qsl, state_slots, counts, H, D, Dv, decay, out, tile_seq, tile_q0, num_tiles, ws, 0, zs,  \
+                         DR, out_part);                                                                                              \
       hipLaunchKernelGGL(lightning_prefix_kernel, dim3(seqs, H, zs), dim3(64), 0, stream, state, ws, positions, qsl, state_slots,    \
                          counts, H, D, Dv, decay);                                                                                   \
-      hipLaunchKernelGGL((lightning_scan_kernel<A, DM, 2>), dim3(num_tiles, H, zs), dim3(64), 0, stream, (const A*)qkvg, row_stride,  \
-                         state, positions, qsl, state_slots, counts, H, D, Dv, decay, out, tile_seq, tile_q0, num_tiles, ws, 0);     \
+      hipLaunchKernelGGL((lightning_scan_kernel<A, DM, 2>), dim3(num_tiles, H, gz), dim3(64), 0, stream, (const A*)qkvg, row_stride,  \
+                         state, positions, qsl, state_slots, counts, H, D, Dv, decay, out, tile_seq, tile_q0, num_tiles, ws, 0, zs,  \
+                         DR, out_part);                                                                                              \
     }                                                                                                                                \
   })
-  if (D <= 32) SM_SCAN(32);
-  else if (D <= 64) SM_SCAN(64);
-  else if (D <= 128) SM_SCAN(128);
+  if (DR <= 32) SM_SCAN(32);
+  else if (DR <= 64) SM_SCAN(64);
+  else if (DR <= 128) SM_SCAN(128);
   else SM_SCAN(256);
 #undef SM_SCAN
 }

@@ -93,15 +93,17 @@ Tensor sm_add_ln(Tensor x, const Tensor& y, const Tensor& w, const Tensor& b, do
 
 Tensor sm_rms_gate(const Tensor& o, const Tensor& w, double eps, const Tensor& gate, bool out_bf16) {
   check_f32(o, "o");
-  TORCH_CHECK(o.dim() == 2, "o must be [T, N]");
-  const int64_t T = o.size(0), N = o.size(1);
+  TORCH_CHECK(o.dim() == 2 || o.dim() == 3, "o must be [T, N] or planes of partial sums [parts, T, N]");
+  const int64_t parts = o.dim() == 3 ? o.size(0) : 1;
+  const int64_t T = o.size(-2), N = o.size(-1);
+  TORCH_CHECK(N * 4 <= kSmMaxLds, "row too wide");
   check_f32(w, "w", N);
   const bool gbf = act_bf16(gate, "gate");
   check_rows(gate, "gate");
   TORCH_CHECK(gate.size(0) == T && gate.size(1) == N, "gate must be [T, N]");
   Tensor out = at::empty({T, N}, o.options().dtype(out_bf16 ? at::kBFloat16 : at::kFloat));
-  dli::launch_sm_rms_gate(o.data_ptr<float>(), w.data_ptr<float>(), (float)eps, gate.data_ptr(), gbf, gate.stride(0), (int)T, (int)N,
-                          out.data_ptr(), out_bf16, cur_stream(o));
+  dli::launch_sm_rms_gate(o.data_ptr<float>(), (int)parts, w.data_ptr<float>(), (float)eps, gate.data_ptr(), gbf, gate.stride(0), (int)T,
+                          (int)N, out.data_ptr(), out_bf16, cur_stream(o));
   return out;
 }
 
@@ -277,7 +279,9 @@ Tensor sm_lightning_scan(const Tensor& qkvg, Tensor state, const Tensor& positio
   check_i32(counts, "counts");
   TORCH_CHECK(positions.numel() >= T && counts.numel() >= 4 && num_seqs >= 0 && qsl.numel() >= num_seqs + 1 &&
                   state_slots.numel() >= num_seqs, "step metadata shorter than the batch");
-  Tensor out = at::zeros({T, H * Dv}, qkvg.options().dtype(at::kFloat));
+  // one plane of partial outputs per part of the state rows (summed by sm_rms_gate)
+  const int64_t parts = dli::sm_lightning_parts((int)D);
+  Tensor out = at::zeros({parts, T, H * Dv}, qkvg.options().dtype(at::kFloat));
   // block path of prefill chunks: 64-token blocks = the step's prefill tiles; one [H, D, Dv] workspace row per block
   const int* ts = nullptr;
   const int* tq = nullptr;
@@ -293,7 +297,7 @@ Tensor sm_lightning_scan(const Tensor& qkvg, Tensor state, const Tensor& positio
   }
   dli::launch_sm_lightning_scan(qkvg.data_ptr(), bf, qkvg.stride(0), state.data_ptr<float>(), positions.data_ptr<int>(),
                                 qsl.data_ptr<int>(), state_slots.data_ptr<int>(), counts.data_ptr<int>(), (int)num_seqs, (int)H, (int)D,
-                                (int)Dv, decay.data_ptr<float>(), out.data_ptr<float>(), ts, tq, (int)num_tiles,
+                                (int)Dv, decay.data_ptr<float>(), out.data_ptr<float>(), T * H * Dv, ts, tq, (int)num_tiles,
                                 num_tiles > 0 ? ws.data_ptr<float>() : nullptr, cur_stream(qkvg));
   return out;
 }

@@ -100,7 +100,8 @@ def add_ln(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, b: torch.Tensor, e
 
 
 def rms_gate(o: torch.Tensor, w: torch.Tensor, eps: float, gate: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    """``o / rms(o) · w · sigmoid(gate)`` per row (``o`` fp32 ``[T, N]``; ``gate`` a row-strided view)."""
+    """``o / rms(o) · w · sigmoid(gate)`` per row (``o`` fp32 ``[T, N]``, or — what the GPU scan returns — planes of partial
+    sums ``[parts, T, N]`` whose sum is the row; ``gate`` a row-strided view)."""
     if o.is_cuda:
         return _hip().sm_rms_gate(o, w, eps, gate, out_dtype == torch.bfloat16)
     y = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps) * w
@@ -242,7 +243,8 @@ def token_attention(out: torch.Tensor, q1: torch.Tensor, q2: Optional[torch.Tens
 def lightning_scan(qkvg: torch.Tensor, state: torch.Tensor, meta, H: int, D: int, Dv: int, decay: torch.Tensor) -> torch.Tensor:
     """``qkvg [T, 2·H·D + 2·H·Dv]`` = ``[q | k | v | gate]`` (pre-activation; the gate columns are not read).  Per sequence
     and head, token by token: ``S ← decay[h] · S + silu(k) silu(v)ᵀ``, ``o = Sᵀ silu(q)`` with ``S`` = the sequence's fp32
-    ``state[slot, h]`` ``[D, Dv]`` (zero at position 0), written back after the step's last token.  Returns fp32 ``[T, H·Dv]``."""
+    ``state[slot, h]`` ``[D, Dv]`` (zero at position 0), written back after the step's last token.  Returns fp32 ``[T, H·Dv]`` (GPU: ``[parts, T, H·Dv]``
+    partial sums over parts of the state rows, for ``rms_gate``)."""
     if _act_ok(qkvg):
         # prefill chunks run block-parallel over the step's 64-token tiles (local states → prefix over blocks → outputs)
         tiles = meta.num_prefill_tiles if BLOCK_SCAN else 0
