@@ -356,7 +356,8 @@ __global__ __launch_bounds__(NT) void token_attention_kernel(
     const A* __restrict__ q2, int64_t q2_ts, int64_t q2_hs, int D2, const A* __restrict__ kc, int rowk,
     const A* __restrict__ vc, int rowv, int vhead, int Dv, const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ positions, const int* __restrict__ token_seq, int H, int G, float scale, int window,
-    const float* __restrict__ temp, const float* __restrict__ r1, const float* __restrict__ r2) {
+    const float* __restrict__ temp, const float* __restrict__ r1, const float* __restrict__ r2, int nsplit,
+    float* __restrict__ part) {
   extern __shared__ float sh[];          // q [HG][Dk] | acc [4 waves][HG][Dv] | m [4][HG] | l [4][HG]
   constexpr int NW = NT / 64;
   const int64_t t = blockIdx.x;
@@ -401,7 +402,13 @@ __global__ __launch_bounds__(NT) void token_attention_kernel(
     for (int v = 0; v < VPL; ++v) acc[hh][v] = 0.f;
   }
 
-  for (int base = lo + wave * 64; base <= p; base += NW * 64) {
+  // gridDim.z = nsplit workgroups share a long key range: each takes a contiguous run of 64-key chunks and leaves
+  // (max, sum, unnormalised output) in `part`; token_attention_merge_kernel combines them
+  const int nchunks = (p - lo + 64) >> 6;
+  const int per_split = (nchunks + nsplit - 1) / nsplit;
+  const int c_begin = blockIdx.z * per_split, c_end = min(c_begin + per_split, nchunks);
+  for (int ci = c_begin + wave; ci < c_end; ci += NW) {
+    const int base = lo + ci * 64;
     const int j = base + lane;
     const bool valid = j <= p;
     int slot = 0;
@@ -414,6 +421,20 @@ __global__ __launch_bounds__(NT) void token_attention_kernel(
       constexpr int KV = 16 / esz;       // elements per 16-byte piece
       int i = 0;
       if (kwide) {
+        for (; i + 2 * KV <= Dk; i += 2 * KV) {          // two 16-byte pieces in flight
+          float kv[2][KV];
+#pragma unroll
+          for (int c4 = 0; c4 < 2; ++c4) load_vals<A, KV == 8 ? 8 : 4>(kr + i + c4 * KV, true, kv[c4]);
+#pragma unroll
+          for (int hh = 0; hh < HG; ++hh) {
+            float d = 0.f;
+#pragma unroll
+            for (int c4 = 0; c4 < 2; ++c4)
+#pragma unroll
+              for (int u = 0; u < KV; ++u) d += qs[hh * Dk + i + c4 * KV + u] * kv[c4][u];
+            s[hh] += d;
+          }
+        }
         for (; i + KV <= Dk; i += KV) {
           float kv[KV];
           load_vals<A, KV == 8 ? 8 : 4>(kr + i, true, kv);
@@ -447,7 +468,27 @@ __global__ __launch_bounds__(NT) void token_attention_kernel(
     }
     const int nvalid = min(p - base + 1, 64);
     if (e0 < Dv) {
-      for (int jj = 0; jj < nvalid; ++jj) {
+      int jj = 0;
+      if (vwide) {
+        constexpr int UB = VPL >= 8 ? 2 : (VPL >= 4 ? 4 : 8);   // value rows fetched together
+        for (; jj + UB <= nvalid; jj += UB) {
+          float vv[UB][VPL];
+#pragma unroll
+          for (int u = 0; u < UB; ++u) {
+            const int sj = __builtin_amdgcn_readlane(slot, jj + u);
+            load_vals<A, VPL>(vc + (int64_t)sj * rowv + g * vhead + e0, true, vv[u]);
+          }
+#pragma unroll
+          for (int u = 0; u < UB; ++u)
+#pragma unroll
+            for (int hh = 0; hh < HG; ++hh) {
+              const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pl[hh]), jj + u));
+#pragma unroll
+              for (int v = 0; v < VPL; ++v) acc[hh][v] += pj * vv[u][v];
+            }
+        }
+      }
+      for (; jj < nvalid; ++jj) {
         const int sj = __builtin_amdgcn_readlane(slot, jj);
         float vv[VPL];
         const A* vr = vc + (int64_t)sj * rowv + g * vhead + e0;
@@ -485,11 +526,47 @@ __global__ __launch_bounds__(NT) void token_attention_kernel(
     float L = 0.f, o = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
-      const float f = expf(ms[w * HG + hh] - M);
+      const float f = M == -INFINITY ? 0.f : expf(ms[w * HG + hh] - M);     // a split without keys: all waves empty
       L += f * ls[w * HG + hh];
       o += f * accs[(w * HG + hh) * Dv + e];
     }
-    stf<A>(out + t * o_ts + (h0 + hh) * o_hs + e, o / L);
+    if (nsplit == 1) {
+      stf<A>(out + t * o_ts + (h0 + hh) * o_hs + e, o / L);
+    } else {
+      float* pr = part + ((t * H + (h0 + hh)) * nsplit + blockIdx.z) * (int64_t)(Dv + 2);
+      pr[2 + e] = o;
+      if (e == 0) {
+        pr[0] = M;
+        pr[1] = L;
+      }
+    }
+  }
+}
+
+// combine the nsplit partial results of a (token, head): part [T][H][nsplit][2 + Dv] = (max, sum, unnormalised output)
+template <typename A>
+__global__ __launch_bounds__(64) void token_attention_merge_kernel(A* __restrict__ out, int64_t o_ts, int64_t o_hs,
+                                                                   const float* __restrict__ part,
+                                                                   const int* __restrict__ token_seq, int H, int Dv,
+                                                                   int nsplit) {
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y;
+  if (token_seq[t] < 0) return;
+  const float* pr = part + (t * H + h) * nsplit * (int64_t)(Dv + 2);
+  float M = -INFINITY;
+  for (int z = 0; z < nsplit; ++z) M = fmaxf(M, pr[z * (Dv + 2)]);
+  float L = 0.f;
+  for (int z = 0; z < nsplit; ++z) {
+    const float mz = pr[z * (Dv + 2)];
+    if (mz != -INFINITY) L += expf(mz - M) * pr[z * (Dv + 2) + 1];
+  }
+  for (int e = threadIdx.x; e < Dv; e += 64) {
+    float o = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+      const float mz = pr[z * (Dv + 2)];
+      if (mz != -INFINITY) o += expf(mz - M) * pr[z * (Dv + 2) + 2 + e];
+    }
+    stf<A>(out + t * o_ts + h * o_hs + e, o / L);
   }
 }
 
@@ -552,9 +629,12 @@ __global__ __launch_bounds__(NT) void tile_attention_kernel(
                  : *reinterpret_cast<const bf16x8*>(q2 + tq * q2_ts + h * q2_hs + (d - D1));
     qf[s] = v;
   }
-  const float qmul = scale * (temp != nullptr ? temp[h] : 1.f);
-  const bool pen = r1 != nullptr;
-  const float r1h = pen ? r1[h] : 0.f, r2h = pen ? r2[h] : 0.f;
+  // scores are kept in the log2 domain: s·log2(e) − r1·log2(1 + r2·distance), weights 2^(s − max) — one v_exp_f32 and one
+  // v_log_f32 per score (this kernel is bound by the per-score vector arithmetic, not by the matrix cores; its results are
+  // rounded to bf16 anyway: the fp32 model never takes this path)
+  const float qmul = scale * (temp != nullptr ? temp[h] : 1.f) * 1.4426950408889634f;
+  const float r1h = r1 != nullptr ? r1[h] : 0.f, r2h = r1 != nullptr ? r2[h] : 0.f;
+  const bool pen = r1h != 0.f;
   const int pq = p0 + q0 + qi;                            // this lane's query position
   const int p_first = p0 + q0, p_last = p0 + q0 + nq - 1;
   const int kb_lo = (window > 0 ? max(p_first - window + 1, 0) : 0) >> 5, kb_hi = p_last >> 5;
@@ -595,26 +675,31 @@ __global__ __launch_bounds__(NT) void tile_attention_kernel(
     }
     float sv[8];
     float mx = -INFINITY;
+    // a page every query of the tile sees whole (the common case far from the diagonal) needs no per-score masks
+    const bool whole = nq == 64 && 32 * kb + 31 <= p_first && (window <= 0 || 32 * kb > p_last - window);
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
       const int j = 32 * kb + (r < 4 ? 4 * g4 + r : 16 + 4 * g4 + (r - 4));
-      const bool ok = qvalid && j <= pq && (window <= 0 || j > pq - window);
       float v = (r < 4 ? sa[r] : sb[r - 4]) * qmul;
-      if (pen) v -= r1h * log1pf(r2h * (float)(pq - j));
-      sv[r] = ok ? v : -INFINITY;
-      mx = fmaxf(mx, sv[r]);
+      if (pen) v -= r1h * __builtin_amdgcn_logf(1.f + r2h * (float)max(pq - j, 0));
+      if (!whole) {
+        const bool ok = qvalid && j <= pq && (window <= 0 || j > pq - window);
+        v = ok ? v : -INFINITY;
+      }
+      sv[r] = v;
+      mx = fmaxf(mx, v);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float mn = fmaxf(m, mx);
     const float mu = mn == -INFINITY ? 0.f : mn;          // nothing visible yet: keep everything at zero
-    const float corr = expf(m - mu);
+    const float corr = fast_exp2(m - mu);
     m = mn;
     bf16x8 ph, plo;
     float ps = 0.f;
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
-      const float pv = expf(sv[r] - mu);
+      const float pv = fast_exp2(sv[r] - mu);
       ps += pv;
       const uint16_t hi = f2bf(pv);
       ph[r] = (short)hi;
@@ -763,7 +848,9 @@ __global__ __launch_bounds__(64) void lightning_prefix_kernel(float* __restrict_
   const int slot = state_slots[seq];
   if (slot < 0 || n < 2) return;
   const int h = blockIdx.y;
-  const int e = blockIdx.z * 64 + threadIdx.x;
+  const int zs = (Dv + 63) >> 6;
+  const int d = blockIdx.z / zs;                       // grid.z = D · (64-column slices): the walk over blocks is per state row
+  const int e = (blockIdx.z - d * zs) * 64 + threadIdx.x;
   if (e >= Dv) return;
   const float lam = decay[h];
   float lam64 = lam;
@@ -774,17 +861,15 @@ __global__ __launch_bounds__(64) void lightning_prefix_kernel(float* __restrict_
   for (int i = 0; i < rest; ++i) lamr *= lam;
   const bool carry = positions[t0] > 0;
   const int blocks = (n + 63) >> 6;
-  float* srow = state + ((int64_t)slot * H + h) * D * Dv + e;
-  for (int d = 0; d < D; ++d) {
-    float run = carry ? srow[(int64_t)d * Dv] : 0.f;
-    for (int i = 0; i < blocks; ++i) {
-      float* w = ws + (((int64_t)(((t0 + 64 * i) >> 6) + seq) * H + h) * D + d) * Dv + e;
-      const float own = *w;
-      *w = run;
-      run = ((i == blocks - 1 && rest) ? lamr : lam64) * run + own;
-    }
-    srow[(int64_t)d * Dv] = run;
+  float* srow = state + (((int64_t)slot * H + h) * D + d) * Dv + e;
+  float run = carry ? *srow : 0.f;
+  for (int i = 0; i < blocks; ++i) {
+    float* w = ws + (((int64_t)(((t0 + 64 * i) >> 6) + seq) * H + h) * D + d) * Dv + e;
+    const float own = *w;
+    *w = run;
+    run = ((i == blocks - 1 && rest) ? lamr : lam64) * run + own;
   }
+  *srow = run;
 }
 
 }  // namespace
@@ -872,11 +957,11 @@ static void token_attention_hg(int hg, dim3 grid, size_t lds, hipStream_t stream
                                int64_t q1_ts, int64_t q1_hs, int D1, const A* q2, int64_t q2_ts, int64_t q2_hs, int D2, const A* kc,
                                int rowk, const A* vc, int rowv, int vhead, int Dv, const int* bt, int max_blocks, const int* pos,
                                const int* tseq, int H, int G, float scale, int window, const float* temp, const float* r1,
-                               const float* r2) {
+                               const float* r2, int nsplit, float* part) {
 #define SM_ATT(HGV)                                                                                                              \
   hipLaunchKernelGGL((token_attention_kernel<A, VPL, HGV>), grid, dim3(NT), lds, stream, out, o_ts, o_hs, q1, q1_ts, q1_hs, D1,  \
                      q2, q2_ts, q2_hs, D2, kc, rowk, vc, rowv, vhead, Dv, bt, max_blocks, pos, tseq, H, G, scale, window, temp,  \
-                     r1, r2)
+                     r1, r2, nsplit, part)
   if (hg == 1) SM_ATT(1);
   else if (hg == 2) SM_ATT(2);
   else SM_ATT(4);
@@ -887,7 +972,7 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
                                const void* q2, int64_t q2_ts, int64_t q2_hs, int D2, const void* kc, int rowk, const void* vc,
                                int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* positions,
                                const int* token_seq, int rows, int H, int G, float scale, int window, const float* temp,
-                               const float* r1, const float* r2, bool bf16, hipStream_t stream) {
+                               const float* r1, const float* r2, bool bf16, int nsplit, float* part, hipStream_t stream) {
   if (rows == 0) return;
   // heads per workgroup: as many of the heads sharing a key / value head as divide their number and fit the LDS budget
   const int per = H / G, Dk = D1 + D2;
@@ -895,18 +980,29 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
   auto lds_of = [&](int g) { return (size_t)(g * Dk + (NT / 64) * g * Dv + 2 * (NT / 64) * g) * sizeof(float); };
   while (hg > 1 && lds_of(hg) > 60 * 1024) hg >>= 1;
   const size_t lds = lds_of(hg);
-  const dim3 grid(rows, H / hg);
+  const dim3 grid(rows, H / hg, nsplit);
   const int nv = (Dv + 63) / 64;
 #define SM_ATT_V(VPLV)                                                                                                            \
   SM_DISPATCH_BF16(bf16, A, (token_attention_hg<A, VPLV>(hg, grid, lds, stream, (A*)out, o_ts, o_hs, (const A*)q1, q1_ts, q1_hs, \
                                                          D1, (const A*)q2, q2_ts, q2_hs, D2, (const A*)kc, rowk, (const A*)vc,   \
                                                          rowv, vhead, Dv, block_tables, max_blocks, positions, token_seq, H, G,  \
-                                                         scale, window, temp, r1, r2)))
+                                                         scale, window, temp, r1, r2, nsplit, part)))
   if (nv <= 1) SM_ATT_V(1);
   else if (nv <= 2) SM_ATT_V(2);
   else if (nv <= 4) SM_ATT_V(4);
   else SM_ATT_V(8);
 #undef SM_ATT_V
+  if (nsplit > 1)
+    SM_DISPATCH_BF16(bf16, A, hipLaunchKernelGGL(token_attention_merge_kernel<A>, dim3(rows, H), dim3(64), 0, stream, (A*)out, o_ts,
+                                                 o_hs, (const float*)part, token_seq, H, Dv, nsplit));
+}
+
+// workgroups of a per-token attention launch over `rows` tokens: long key ranges are cut so that about 1024 exist
+int sm_token_attention_splits(int rows, int H, int G) {
+  const int per = H / G;
+  const int hg = per % 4 == 0 ? 4 : (per % 2 == 0 ? 2 : 1);
+  const int wgs = std::max(rows * (H / hg), 1);
+  return std::max(1, std::min(8, 1024 / wgs));
 }
 
 // prefill tiles on the matrix cores (bf16; see tile_attention_kernel).  Returns false when the shapes do not fit its
@@ -968,7 +1064,7 @@ void launch_sm_lightning_scan(const void* qkvg, bool bf16, int64_t row_stride, f
       hipLaunchKernelGGL((lightning_scan_kernel<A, DM, 1>), dim3(num_tiles, H, gz), dim3(64), 0, stream, (const A*)qkvg, row_stride,  \
                          state, positions, qsl, state_slots, counts, H, D, Dv, decay, out, tile_seq, tile_q0, num_tiles, ws, 0, zs,  \
                          DR, out_part);                                                                                              \
-      hipLaunchKernelGGL(lightning_prefix_kernel, dim3(seqs, H, zs), dim3(64), 0, stream, state, ws, positions, qsl, state_slots,    \
+      hipLaunchKernelGGL(lightning_prefix_kernel, dim3(seqs, H, zs * D), dim3(64), 0, stream, state, ws, positions, qsl, state_slots, \
                          counts, H, D, Dv, decay);                                                                                   \
       hipLaunchKernelGGL((lightning_scan_kernel<A, DM, 2>), dim3(num_tiles, H, gz), dim3(64), 0, stream, (const A*)qkvg, row_stride,  \
                          state, positions, qsl, state_slots, counts, H, D, Dv, decay, out, tile_seq, tile_q0, num_tiles, ws, 0, zs,  \

@@ -201,12 +201,18 @@ void sm_token_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor
   TORCH_CHECK(block_tables.dim() == 2 && positions.numel() >= T && token_seq.numel() >= T, "step metadata shorter than the batch");
   TORCH_CHECK(r1.has_value() == r2.has_value(), "r1 and r2 come together");
   TORCH_CHECK((Dk + 4 * Dv + 8) * 4 <= kSmMaxLds, "head sizes exceed the kernel's LDS budget");
+  // few rows (decode steps): long key ranges are cut over several workgroups, partial results in `part`
+  const int64_t n_rows = rows < 0 ? T : rows;
+  const int nsplit = dli::sm_token_attention_splits((int)n_rows, (int)H, (int)G);
+  Tensor part;
+  if (nsplit > 1) part = at::empty({n_rows, H, nsplit, Dv + 2}, q1.options().dtype(at::kFloat));
   dli::launch_sm_token_attention(out.data_ptr(), out.stride(0), out.stride(1), q1.data_ptr(), q1.stride(0), q1.stride(1), (int)D1,
                                  q2.has_value() ? q2->data_ptr() : nullptr, q2.has_value() ? q2->stride(0) : 0,
                                  q2.has_value() ? q2->stride(1) : 0, (int)D2, k_cache.data_ptr(), (int)(G * Dk), vc.data_ptr(),
                                  (int)vc.size(2), (int)vhead, (int)Dv, block_tables.data_ptr<int>(), (int)block_tables.size(1),
-                                 positions.data_ptr<int>(), token_seq.data_ptr<int>(), (int)(rows < 0 ? T : rows), (int)H, (int)G, (float)scale,
-                                 (int)window, opt_f32(temp, "temp", H), opt_f32(r1, "r1", H), opt_f32(r2, "r2", H), bf, cur_stream(q1));
+                                 positions.data_ptr<int>(), token_seq.data_ptr<int>(), (int)n_rows, (int)H, (int)G, (float)scale,
+                                 (int)window, opt_f32(temp, "temp", H), opt_f32(r1, "r1", H), opt_f32(r2, "r2", H), bf, nsplit,
+                                 nsplit > 1 ? part.data_ptr<float>() : nullptr, cur_stream(q1));
 }
 
 // Prefill tiles (64 queries of one sequence's chunk each) on the matrix cores; bf16 only.  False: shapes the tile kernel does
