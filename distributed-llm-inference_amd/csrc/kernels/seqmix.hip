@@ -579,8 +579,8 @@ __global__ __launch_bounds__(64) void token_attention_merge_kernel(A* __restrict
 // remainder (two MFMAs: P enters the product with 16 mantissa bits, not 8).  The lane's eight Sᵀ values (two 16-key
 // tiles) are, in register order, the B fragment of the P·V k-step when the staged V columns sit in the slot order
 // slot(t) = ((t & 15) >> 2)·8 + (t >> 4)·4 + (t & 3).  KSMAX / MTMAX: compile-time bounds of ceil(Dk / 32) and Dv / 16.
-template <int KSMAX, int MTMAX>
-__global__ __launch_bounds__(NT) void tile_attention_kernel(
+template <int KSMAX, int MTMAX, int HW>
+__global__ __launch_bounds__(NT * HW) void tile_attention_kernel(
     uint16_t* __restrict__ out, int64_t o_ts, int64_t o_hs, const uint16_t* __restrict__ q1, int64_t q1_ts, int64_t q1_hs, int D1,
     const uint16_t* __restrict__ q2, int64_t q2_ts, int64_t q2_hs, int D2, const uint16_t* __restrict__ kc, int rowk,
     const uint16_t* __restrict__ vc, int rowv, int vhead, int Dv, const int* __restrict__ block_tables, int max_blocks,
@@ -592,14 +592,17 @@ __global__ __launch_bounds__(NT) void tile_attention_kernel(
   // the host walks causal tiles longest-first from the END of the list
   const int tile = num_tiles - 1 - (int)blockIdx.x;
   if (tile >= ntiles) return;
-  const int h = blockIdx.y;
+  // HW heads of one key / value group per workgroup (4 waves each): the staged page serves all of them
+  constexpr int TNT = NT * HW;
+  const int wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int h = blockIdx.y * HW + (wave_all >> 2);
   const int seq = tile_seq[tile], q0 = tile_q0[tile];
   const int t_begin = qsl[seq];
   const int n_chunk = qsl[seq + 1] - t_begin;
   const int p0 = seq_lens[seq] - n_chunk;                 // position of the chunk's first token
   const int nq = min(64, n_chunk - q0);
   if (nq <= 0) return;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave = wave_all & 3;
   const int lane = threadIdx.x & 63, g4 = lane >> 4, c = lane & 15;
   const int Dk = D1 + D2;
   const int KS = (Dk + 31) >> 5, MT = Dv >> 4;
@@ -610,7 +613,7 @@ __global__ __launch_bounds__(NT) void tile_attention_kernel(
   const int g = h / (H / G);
 
   // zero the K padding columns once (Dk not a multiple of 32): they are never staged over
-  for (int i = threadIdx.x; i < 32 * (KS * 32 - Dk); i += NT) {
+  for (int i = threadIdx.x; i < 32 * (KS * 32 - Dk); i += TNT) {
     const int row = i / (KS * 32 - Dk), col = Dk + i % (KS * 32 - Dk);
     Ks[row * KST + col] = 0;
   }
@@ -649,12 +652,12 @@ __global__ __launch_bounds__(NT) void tile_attention_kernel(
   for (int kb = kb_lo; kb <= kb_hi; ++kb) {
     __syncthreads();                                      // everyone is done with the previous page
     const int64_t page_row = (int64_t)bt[kb] * kBlockTokens;
-    for (int i = threadIdx.x; i < 32 * kchunks; i += NT) {
+    for (int i = threadIdx.x; i < 32 * kchunks; i += TNT) {
       const int row = i / kchunks, ch = i - row * kchunks;
       *reinterpret_cast<bf16x8*>(Ks + row * KST + 8 * ch) =
           *reinterpret_cast<const bf16x8*>(kc + (page_row + row) * rowk + g * Dk + 8 * ch);
     }
-    for (int i = threadIdx.x; i < 32 * vchunks; i += NT) {
+    for (int i = threadIdx.x; i < 32 * vchunks; i += TNT) {
       const int row = i & 31, ch = i >> 5;
       const bf16x8 v = *reinterpret_cast<const bf16x8*>(vc + (page_row + row) * rowv + g * vhead + 8 * ch);
       const int slot = ((row & 15) >> 2) * 8 + (row >> 4) * 4 + (row & 3);
@@ -974,6 +977,15 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
                                const int* token_seq, int rows, int H, int G, float scale, int window, const float* temp,
                                const float* r1, const float* r2, bool bf16, int nsplit, float* part, hipStream_t stream) {
   if (rows == 0) return;
+  if (Dv > 512) {
+    // wider values than a lane's 8 columns × 64 lanes: slabs of 512 columns, each a launch of its own (scores recomputed)
+    for (int e = 0; e < Dv; e += 512)
+      launch_sm_token_attention(bf16 ? (void*)((uint16_t*)out + e) : (void*)((float*)out + e), o_ts, o_hs, q1, q1_ts, q1_hs, D1, q2,
+                                q2_ts, q2_hs, D2, kc, rowk, bf16 ? (const void*)((const uint16_t*)vc + e) : (const void*)((const float*)vc + e),
+                                rowv, vhead, std::min(512, Dv - e), block_tables, max_blocks, positions, token_seq, rows, H, G, scale,
+                                window, temp, r1, r2, bf16, 1, nullptr, stream);
+    return;
+  }
   // heads per workgroup: as many of the heads sharing a key / value head as divide their number and fit the LDS budget
   const int per = H / G, Dk = D1 + D2;
   int hg = per % 4 == 0 ? 4 : (per % 2 == 0 ? 2 : 1);
@@ -1021,24 +1033,32 @@ bool launch_sm_tile_attention(void* out, int64_t o_ts, int64_t o_hs, const void*
   if (!ok) return false;
   if (num_tiles == 0) return true;
   const size_t lds = (size_t)(32 * (KS * 32 + 8) + Dv * 40) * sizeof(uint16_t);
-  const dim3 grid(num_tiles, H);
-#define SM_TILE(KSM, MTM)                                                                                                        \
+  // two heads of a key / value group per workgroup (8 waves) where the group has an even number of heads
+  const int hw = (H / G) % 2 == 0 ? 2 : 1;
+  const dim3 grid(num_tiles, H / hw);
+#define SM_TILE_HW(KSM, MTM, HWV)                                                                                                \
   do {                                                                                                                           \
     static bool big = false;                                                                                                     \
     if (lds > 48 * 1024 && !big) {                                                                                               \
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&tile_attention_kernel<KSM, MTM>),                                 \
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&tile_attention_kernel<KSM, MTM, HWV>),                            \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);                                         \
       big = true;                                                                                                                \
     }                                                                                                                            \
-    hipLaunchKernelGGL((tile_attention_kernel<KSM, MTM>), grid, dim3(NT), lds, stream, (uint16_t*)out, o_ts, o_hs,               \
+    hipLaunchKernelGGL((tile_attention_kernel<KSM, MTM, HWV>), grid, dim3(NT * HWV), lds, stream, (uint16_t*)out, o_ts, o_hs,    \
                        (const uint16_t*)q1, q1_ts, q1_hs, D1, (const uint16_t*)q2, q2_ts, q2_hs, D2, (const uint16_t*)kc, rowk,  \
                        (const uint16_t*)vc, rowv, vhead, Dv, block_tables, max_blocks, seq_lens, qsl, tile_seq, tile_q0,        \
                        num_tiles, counts, H, G, scale, window, temp, r1, r2);                                                    \
+  } while (0)
+#define SM_TILE(KSM, MTM)              \
+  do {                                 \
+    if (hw == 2) SM_TILE_HW(KSM, MTM, 2); \
+    else SM_TILE_HW(KSM, MTM, 1);      \
   } while (0)
   if (KS <= 4 && MT <= 8) SM_TILE(4, 8);
   else if (KS <= 8 && MT <= 16) SM_TILE(8, 16);
   else SM_TILE(18, 32);
 #undef SM_TILE
+#undef SM_TILE_HW
   return true;
 }
 

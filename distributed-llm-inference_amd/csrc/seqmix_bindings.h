@@ -192,7 +192,7 @@ void sm_token_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor
   } else {
     TORCH_CHECK(Dv <= Dk, "values read from the key rows cannot be wider than a key");
   }
-  TORCH_CHECK(Dv > 0 && Dv <= 512, "value size must be in 1..512");
+  TORCH_CHECK(Dv > 0 && Dv <= 8192, "value size must be in 1..8192");
   TORCH_CHECK(out.is_cuda() && out.scalar_type() == q1.scalar_type() && out.dim() == 3 && out.stride(2) == 1 && out.size(0) == T &&
                   out.size(1) == H && out.size(2) == Dv, "out must be [T, H, Dv]");
   check_i32(block_tables, "block_tables");
@@ -200,10 +200,10 @@ void sm_token_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor
   check_i32(token_seq, "token_seq");
   TORCH_CHECK(block_tables.dim() == 2 && positions.numel() >= T && token_seq.numel() >= T, "step metadata shorter than the batch");
   TORCH_CHECK(r1.has_value() == r2.has_value(), "r1 and r2 come together");
-  TORCH_CHECK((Dk + 4 * Dv + 8) * 4 <= kSmMaxLds, "head sizes exceed the kernel's LDS budget");
+  TORCH_CHECK((Dk + 4 * std::min<int64_t>(Dv, 512) + 8) * 4 <= kSmMaxLds, "head sizes exceed the kernel's LDS budget");
   // few rows (decode steps): long key ranges are cut over several workgroups, partial results in `part`
   const int64_t n_rows = rows < 0 ? T : rows;
-  const int nsplit = dli::sm_token_attention_splits((int)n_rows, (int)H, (int)G);
+  const int nsplit = Dv > 512 ? 1 : dli::sm_token_attention_splits((int)n_rows, (int)H, (int)G);
   Tensor part;
   if (nsplit > 1) part = at::empty({n_rows, H, nsplit, Dv + 2}, q1.options().dtype(at::kFloat));
   dli::launch_sm_token_attention(out.data_ptr(), out.stride(0), out.stride(1), q1.data_ptr(), q1.stride(0), q1.stride(1), (int)D1,
@@ -275,7 +275,7 @@ Tensor sm_lightning_scan(const Tensor& qkvg, Tensor state, const Tensor& positio
   check_rows(qkvg, "qkvg");
   const int64_t T = qkvg.size(0);
   TORCH_CHECK(qkvg.size(1) >= 2 * H * D + H * Dv, "qkvg row narrower than q | k | v");
-  TORCH_CHECK(D > 0 && D <= 256, "key size must be in 1..256");
+  TORCH_CHECK(D > 0 && D <= 1024, "key size must be in 1..1024");     // a wave keeps at most 256 state rows, D is cut in up to 4 parts
   check_f32(state, "state");
   TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == D && state.size(3) == Dv, "state must be [slots, H, D, Dv]");
   check_f32(decay, "decay", H);

@@ -155,7 +155,12 @@ def other_size_configs():
     m1["mlp"] = {"kind": "dense", "ff": 40}
     m2 = copy.deepcopy(LATENT)
     m2["mixer"].update(heads=1, dim=32, rot_dim=16, vdim=64, kv_rank=80, rot={"base": 1e6, "dims": 2})
+    wide = copy.deepcopy(LATENT)
+    wide["mixer"].update(heads=2, dim=8, rot_dim=8, vdim=8, kv_rank=528, rot={"base": 1000.0, "dims": 8})   # latent wider than 512
+    tall = copy.deepcopy(LIGHT)
+    tall["mixer"].update(heads=1, dim=264, vdim=8, decay=[0.97])                                                # more than 256 state rows
     return {
+        "wide latent, tall state": make_cfg([wide, tall], width=40, vocab=50),
         "square heads, long window": make_cfg([a, l1], width=88, vocab=97, mult=1.0, cap=None),
         "single heads, whole stack three times": make_cfg([a1, m2, l2], width=48, vocab=130, loop=(0, 3, 3), eps=1e-3),
         "loop at the end": make_cfg([m1, l2, a], width=56, vocab=64, loop=(2, 3, 2), mult=0.1, cap=3.0),
