@@ -90,6 +90,12 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
                                const int* token_seq, int rows, int H, int G, float scale, int window, const float* temp,
                                const float* r1, const float* r2, bool bf16, int nsplit, float* part, hipStream_t stream);
 int sm_token_attention_splits(int rows, int H, int G);
+bool launch_sm_head_decode_attention(void* out, int64_t o_ts, int64_t o_hs, const void* q1, int64_t q1_ts, int64_t q1_hs, int D1,
+                                     const void* q2, int64_t q2_ts, int64_t q2_hs, int D2, const void* kc, int rowk, const void* vc,
+                                     int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* positions,
+                                     const int* token_seq, int rows, int H, int G, float scale, int window, const float* temp,
+                                     const float* r1, const float* r2, int nsplit, float* part, hipStream_t stream);
+int sm_head_decode_splits(int rows, int H, int G);
 bool launch_sm_tile_attention(void* out, int64_t o_ts, int64_t o_hs, const void* q1, int64_t q1_ts, int64_t q1_hs, int D1,
                               const void* q2, int64_t q2_ts, int64_t q2_hs, int D2, const void* kc, int rowk, const void* vc,
                               int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* seq_lens,

@@ -736,6 +736,167 @@ __global__ __launch_bounds__(NT * HW) void tile_attention_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------------------ attention, decode rows, heads as columns
+// bf16 only; for mixers whose query heads share a key / value head in groups of 8 or more (latent attention: all of them).
+// One workgroup per (token, group of up to 16 heads, slice of the key range): the 16 MFMA columns are the HEADS of one
+// token, so a key row fetched once meets every head on the matrix cores.  Pages are staged as in tile_attention_kernel
+// (K rows, V transposed into the MFMA slot order); all four waves compute the same Sᵀ = K·Qᵀ tile and online softmax, and
+// each accumulates its own quarter of the value columns, so nothing is merged inside the workgroup.  gridDim.z slices of
+// the key range leave (max, sum, unnormalised output) in `part` for token_attention_merge_kernel.
+template <int KSMAX, int MTQ>
+__global__ __launch_bounds__(NT) void head_decode_attention_kernel(
+    uint16_t* __restrict__ out, int64_t o_ts, int64_t o_hs, const uint16_t* __restrict__ q1, int64_t q1_ts, int64_t q1_hs, int D1,
+    const uint16_t* __restrict__ q2, int64_t q2_ts, int64_t q2_hs, int D2, const uint16_t* __restrict__ kc, int rowk,
+    const uint16_t* __restrict__ vc, int rowv, int vhead, int Dv, const int* __restrict__ block_tables, int max_blocks,
+    const int* __restrict__ positions, const int* __restrict__ token_seq, int H, int G, int groups, float scale, int window,
+    const float* __restrict__ temp, const float* __restrict__ r1, const float* __restrict__ r2, int nsplit,
+    float* __restrict__ part) {
+  extern __shared__ __align__(16) uint16_t tl[];
+  const int64_t t = blockIdx.x;
+  const int seq = token_seq[t];
+  if (seq < 0) return;
+  const int per = H / G;
+  const int g = blockIdx.y / groups, grp = blockIdx.y - g * groups;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63, g4 = lane >> 4, c = lane & 15;
+  const bool hvalid = 16 * grp + c < per;
+  const int h = g * per + min(16 * grp + c, per - 1);
+  const int Dk = D1 + D2;
+  const int KS = (Dk + 31) >> 5, MT = Dv >> 4;
+  const int MTW = (MT + 3) >> 2;                         // value tiles per wave
+  const int KST = KS * 32 + 8;
+  constexpr int VST = 40;
+  uint16_t* Ks = tl;
+  uint16_t* Vt = tl + 32 * KST;
+  for (int i = threadIdx.x; i < 32 * (KS * 32 - Dk); i += NT) {
+    const int row = i / (KS * 32 - Dk), col = Dk + i % (KS * 32 - Dk);
+    Ks[row * KST + col] = 0;
+  }
+  bf16x8 qf[KSMAX];
+#pragma unroll
+  for (int s = 0; s < KSMAX; ++s) {
+    const int d = 32 * s + 8 * g4;
+    bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (s < KS && hvalid && d < Dk)
+      v = d < D1 ? *reinterpret_cast<const bf16x8*>(q1 + t * q1_ts + h * q1_hs + d)
+                 : *reinterpret_cast<const bf16x8*>(q2 + t * q2_ts + h * q2_hs + (d - D1));
+    qf[s] = v;
+  }
+  const float qmul = scale * (temp != nullptr ? temp[h] : 1.f) * 1.4426950408889634f;     // log2 domain, as in the tile kernel
+  const float r1h = r1 != nullptr ? r1[h] : 0.f, r2h = r1 != nullptr ? r2[h] : 0.f;
+  const bool pen = r1 != nullptr;
+  const int p = positions[t];
+  const int lo = window > 0 ? max(p - window + 1, 0) : 0;
+  const int kb_lo = lo >> 5, kb_hi = p >> 5;
+  const int per_split = (kb_hi - kb_lo + nsplit) / nsplit;
+  const int kb_begin = kb_lo + blockIdx.z * per_split, kb_end = min(kb_begin + per_split - 1, kb_hi);
+  const int* bt = block_tables + (int64_t)seq * max_blocks;
+
+  float m = -INFINITY, l = 0.f;
+  f32x4 acc[MTQ];
+#pragma unroll
+  for (int i = 0; i < MTQ; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int kchunks = Dk >> 3, vchunks = Dv >> 3;
+  for (int kb = kb_begin; kb <= kb_end; ++kb) {
+    __syncthreads();
+    const int64_t page_row = (int64_t)bt[kb] * kBlockTokens;
+    for (int i = threadIdx.x; i < 32 * kchunks; i += NT) {
+      const int row = i / kchunks, ch = i - row * kchunks;
+      *reinterpret_cast<bf16x8*>(Ks + row * KST + 8 * ch) =
+          *reinterpret_cast<const bf16x8*>(kc + (page_row + row) * rowk + g * Dk + 8 * ch);
+    }
+    for (int i = threadIdx.x; i < 32 * vchunks; i += NT) {
+      const int row = i & 31, ch = i >> 5;
+      const bf16x8 v = *reinterpret_cast<const bf16x8*>(vc + (page_row + row) * rowv + g * vhead + 8 * ch);
+      const int slot = ((row & 15) >> 2) * 8 + (row >> 4) * 4 + (row & 3);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) Vt[(8 * ch + j) * VST + slot] = (uint16_t)v[j];
+    }
+    __syncthreads();
+    f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < KSMAX; ++s) {
+      if (s < KS) {
+        const bf16x8 ka = *reinterpret_cast<const bf16x8*>(Ks + c * KST + 32 * s + 8 * g4);
+        const bf16x8 kb2 = *reinterpret_cast<const bf16x8*>(Ks + (16 + c) * KST + 32 * s + 8 * g4);
+        sa = mfma16(ka, qf[s], sa);
+        sb = mfma16(kb2, qf[s], sb);
+      }
+    }
+    float sv[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int j = 32 * kb + (r < 4 ? 4 * g4 + r : 16 + 4 * g4 + (r - 4));
+      float v = (r < 4 ? sa[r] : sb[r - 4]) * qmul;
+      if (pen) v -= r1h * __builtin_amdgcn_logf(1.f + r2h * (float)max(p - j, 0));
+      v = (j >= lo && j <= p) ? v : -INFINITY;
+      sv[r] = v;
+      mx = fmaxf(mx, v);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mn = fmaxf(m, mx);
+    const float mu = mn == -INFINITY ? 0.f : mn;
+    const float corr = fast_exp2(m - mu);
+    m = mn;
+    bf16x8 ph, plo;
+    float ps = 0.f;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const float pv = fast_exp2(sv[r] - mu);
+      ps += pv;
+      const uint16_t hi = f2bf(pv);
+      ph[r] = (short)hi;
+      plo[r] = (short)f2bf(pv - bf2f(hi));
+    }
+    l = l * corr + ps;
+#pragma unroll
+    for (int ii = 0; ii < MTQ; ++ii) {
+      const int i = wave * MTW + ii;
+      if (ii < MTW && i < MT) {
+        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vt + (16 * i + c) * VST + 8 * g4);
+        f32x4 a = acc[ii];
+        a[0] *= corr; a[1] *= corr; a[2] *= corr; a[3] *= corr;
+        a = mfma16(vf, ph, a);
+        acc[ii] = mfma16(vf, plo, a);
+      }
+    }
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!hvalid) return;
+  if (nsplit == 1) {
+    const float rl = 1.f / l;
+    uint16_t* orow = out + t * o_ts + h * o_hs;
+#pragma unroll
+    for (int ii = 0; ii < MTQ; ++ii) {
+      const int i = wave * MTW + ii;
+      if (ii < MTW && i < MT) {
+        bf16x4 o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = (short)f2bf(acc[ii][r] * rl);
+        *reinterpret_cast<bf16x4*>(orow + 16 * i + 4 * g4) = o;
+      }
+    }
+  } else {
+    // the merge kernel works with natural exponentials: hand it the maximum in that domain
+    float* pr = part + ((t * H + h) * nsplit + blockIdx.z) * (int64_t)(Dv + 2);
+    if (wave == 0 && g4 == 0) {
+      pr[0] = m * 0.6931471805599453f;
+      pr[1] = l;
+    }
+#pragma unroll
+    for (int ii = 0; ii < MTQ; ++ii) {
+      const int i = wave * MTW + ii;
+      if (ii < MTW && i < MT) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) pr[2 + 16 * i + 4 * g4 + r] = acc[ii][r];
+      }
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ linear attention
 // S ← decay·S + silu(k)·silu(v)ᵀ, o = Sᵀ silu(q), token by token, with S = a [D, Dv] fp32 state per (sequence, head).
 // One wave per (work item, head, 64 value columns): lane e keeps column e of the state in registers; the next token's
@@ -1060,6 +1221,52 @@ bool launch_sm_tile_attention(void* out, int64_t o_ts, int64_t o_hs, const void*
 #undef SM_TILE
 #undef SM_TILE_HW
   return true;
+}
+
+// decode rows with heads as MFMA columns (bf16; see head_decode_attention_kernel).  False: shapes it does not take.
+bool launch_sm_head_decode_attention(void* out, int64_t o_ts, int64_t o_hs, const void* q1, int64_t q1_ts, int64_t q1_hs, int D1,
+                                     const void* q2, int64_t q2_ts, int64_t q2_hs, int D2, const void* kc, int rowk, const void* vc,
+                                     int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* positions,
+                                     const int* token_seq, int rows, int H, int G, float scale, int window, const float* temp,
+                                     const float* r1, const float* r2, int nsplit, float* part, hipStream_t stream) {
+  const int Dk = D1 + D2, KS = (Dk + 31) / 32, MT = Dv / 16, per = H / G;
+  auto al = [](const void* p, int64_t a) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % a == 0; };
+  const bool ok = per >= 8 && D1 % 8 == 0 && D2 % 8 == 0 && Dv % 16 == 0 && KS <= 18 && MT <= 32 && rowk % 8 == 0 && rowv % 8 == 0 &&
+                  vhead % 8 == 0 && q1_ts % 8 == 0 && q1_hs % 8 == 0 && q2_ts % 8 == 0 && q2_hs % 8 == 0 && o_ts % 4 == 0 &&
+                  o_hs % 4 == 0 && al(out, 8) && al(q1, 16) && al(q2, 16) && al(kc, 16) && al(vc, 16);
+  if (!ok) return false;
+  if (rows == 0) return true;
+  const size_t lds = (size_t)(32 * (KS * 32 + 8) + Dv * 40) * sizeof(uint16_t);
+  const int groups = (per + 15) / 16;
+  const dim3 grid(rows, G * groups, nsplit);
+#define SM_HD(KSM, MTQV)                                                                                                         \
+  do {                                                                                                                           \
+    static bool big = false;                                                                                                     \
+    if (lds > 48 * 1024 && !big) {                                                                                               \
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&head_decode_attention_kernel<KSM, MTQV>),                         \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);                                         \
+      big = true;                                                                                                                \
+    }                                                                                                                            \
+    hipLaunchKernelGGL((head_decode_attention_kernel<KSM, MTQV>), grid, dim3(NT), lds, stream, (uint16_t*)out, o_ts, o_hs,       \
+                       (const uint16_t*)q1, q1_ts, q1_hs, D1, (const uint16_t*)q2, q2_ts, q2_hs, D2, (const uint16_t*)kc, rowk,  \
+                       (const uint16_t*)vc, rowv, vhead, Dv, block_tables, max_blocks, positions, token_seq, H, G, groups, scale,\
+                       window, temp, r1, r2, nsplit, part);                                                                      \
+  } while (0)
+  if (KS <= 4 && MT <= 8) SM_HD(4, 2);
+  else if (KS <= 8 && MT <= 16) SM_HD(8, 4);
+  else SM_HD(18, 8);
+#undef SM_HD
+  if (nsplit > 1)
+    hipLaunchKernelGGL(token_attention_merge_kernel<uint16_t>, dim3(rows, H), dim3(64), 0, stream, (uint16_t*)out, o_ts, o_hs,
+                       (const float*)part, token_seq, H, Dv, nsplit);
+  return true;
+}
+
+// slices of the key range for that kernel: about 512 workgroups
+int sm_head_decode_splits(int rows, int H, int G) {
+  const int per = H / G;
+  const int wgs = std::max(rows * G * ((per + 15) / 16), 1);
+  return std::max(1, std::min(16, 512 / wgs));
 }
 
 // rows of the state one wave keeps: D is cut into parts so that a wave's per-token loop is short and more waves share the work

@@ -215,6 +215,54 @@ void sm_token_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor
                                  nsplit > 1 ? part.data_ptr<float>() : nullptr, cur_stream(q1));
 }
 
+// Decode rows (the first `rows` tokens) of a mixer whose heads share key / value heads in groups of 8 or more, heads as the
+// MFMA columns; bf16 only.  False: shapes that kernel does not take — nothing was launched.
+bool sm_head_decode_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor>& q2, const Tensor& k_cache,
+                              const c10::optional<Tensor>& v_cache, const Tensor& block_tables, const Tensor& positions,
+                              const Tensor& token_seq, int64_t G, int64_t Dv, double scale, int64_t window,
+                              const c10::optional<Tensor>& temp, const c10::optional<Tensor>& r1, const c10::optional<Tensor>& r2,
+                              int64_t rows) {
+  TORCH_CHECK(q1.is_cuda() && q1.scalar_type() == at::kBFloat16 && q1.dim() == 3 && q1.stride(2) == 1, "q1 must be bfloat16 [T, H, D1]");
+  const int64_t T = q1.size(0), H = q1.size(1), D1 = q1.size(2);
+  TORCH_CHECK(rows >= 0 && rows <= T, "rows past the batch");
+  int64_t D2 = 0;
+  if (q2.has_value()) {
+    TORCH_CHECK(q2->is_cuda() && q2->scalar_type() == at::kBFloat16 && q2->dim() == 3 && q2->stride(2) == 1 && q2->size(0) == T &&
+                    q2->size(1) == H, "q2 must be [T, H, D2] like q1");
+    D2 = q2->size(2);
+  }
+  TORCH_CHECK(G > 0 && H % G == 0, "query heads must be a multiple of the key heads");
+  const int64_t Dk = D1 + D2;
+  TORCH_CHECK(k_cache.is_cuda() && k_cache.is_contiguous() && k_cache.scalar_type() == at::kBFloat16 && k_cache.dim() == 3 &&
+                  k_cache.size(1) == kSmPageTokens && k_cache.size(2) == G * Dk, "k_cache must be [pages, 32, G*(D1+D2)]");
+  const Tensor& vc = v_cache.has_value() ? *v_cache : k_cache;
+  int64_t vhead = Dk;
+  if (v_cache.has_value()) {
+    TORCH_CHECK(vc.is_cuda() && vc.is_contiguous() && vc.scalar_type() == at::kBFloat16 && vc.dim() == 3 && vc.size(0) == k_cache.size(0) &&
+                    vc.size(1) == kSmPageTokens && vc.size(2) == G * Dv, "v_cache must be [pages, 32, G*Dv]");
+    vhead = Dv;
+  } else {
+    TORCH_CHECK(Dv <= Dk, "values read from the key rows cannot be wider than a key");
+  }
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == at::kBFloat16 && out.dim() == 3 && out.stride(2) == 1 && out.size(0) == T &&
+                  out.size(1) == H && out.size(2) == Dv, "out must be [T, H, Dv]");
+  check_i32(block_tables, "block_tables");
+  check_i32(positions, "positions");
+  check_i32(token_seq, "token_seq");
+  TORCH_CHECK(block_tables.dim() == 2 && positions.numel() >= T && token_seq.numel() >= T, "step metadata shorter than the batch");
+  TORCH_CHECK(r1.has_value() == r2.has_value(), "r1 and r2 come together");
+  const int nsplit = dli::sm_head_decode_splits((int)rows, (int)H, (int)G);
+  Tensor part;
+  if (nsplit > 1) part = at::empty({std::max<int64_t>(rows, 1), H, nsplit, Dv + 2}, q1.options().dtype(at::kFloat));
+  return dli::launch_sm_head_decode_attention(out.data_ptr(), out.stride(0), out.stride(1), q1.data_ptr(), q1.stride(0), q1.stride(1),
+                                              (int)D1, q2.has_value() ? q2->data_ptr() : nullptr, q2.has_value() ? q2->stride(0) : 0,
+                                              q2.has_value() ? q2->stride(1) : 0, (int)D2, k_cache.data_ptr(), (int)(G * Dk),
+                                              vc.data_ptr(), (int)vc.size(2), (int)vhead, (int)Dv, block_tables.data_ptr<int>(),
+                                              (int)block_tables.size(1), positions.data_ptr<int>(), token_seq.data_ptr<int>(), (int)rows,
+                                              (int)H, (int)G, (float)scale, (int)window, opt_f32(temp, "temp", H), opt_f32(r1, "r1", H),
+                                              opt_f32(r2, "r2", H), nsplit, nsplit > 1 ? part.data_ptr<float>() : nullptr, cur_stream(q1));
+}
+
 // Prefill tiles (64 queries of one sequence's chunk each) on the matrix cores; bf16 only.  False: shapes the tile kernel does
 // not take — nothing was launched, the caller uses the per-token kernel.
 bool sm_tile_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor>& q2, const Tensor& k_cache,

@@ -593,6 +593,9 @@ TORCH_LIBRARY(dli, m) {
   m.def("sm_token_attention(Tensor(a!) out, Tensor q1, Tensor? q2, Tensor k_cache, Tensor? v_cache, Tensor block_tables, "
         "Tensor positions, Tensor token_seq, int G, int Dv, float scale, int window, Tensor? temp, Tensor? r1, Tensor? r2, int rows=-1) -> ()",
         &sm_token_attention);
+  m.def("sm_head_decode_attention(Tensor(a!) out, Tensor q1, Tensor? q2, Tensor k_cache, Tensor? v_cache, Tensor block_tables, "
+        "Tensor positions, Tensor token_seq, int G, int Dv, float scale, int window, Tensor? temp, Tensor? r1, Tensor? r2, int rows) -> bool",
+        &sm_head_decode_attention);
   m.def("sm_tile_attention(Tensor(a!) out, Tensor q1, Tensor? q2, Tensor k_cache, Tensor? v_cache, Tensor block_tables, Tensor seq_lens, "
         "Tensor qsl, Tensor tile_seq, Tensor tile_q0, int num_tiles, Tensor? counts, int G, int Dv, float scale, int window, "
         "Tensor? temp, Tensor? r1, Tensor? r2) -> bool", &sm_tile_attention);

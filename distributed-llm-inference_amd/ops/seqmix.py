@@ -23,6 +23,7 @@ from ..config import KV_BLOCK_SIZE
 
 
 TILE_ATTENTION = os.environ.get("DLI_TILE_ATTENTION", "1") != "0"     # A/B knob: prefill tiles on the matrix cores (bf16)
+HEAD_DECODE = os.environ.get("DLI_HEAD_DECODE", "1") != "0"           # A/B knob: decode rows of head-sharing mixers on the matrix cores
 BLOCK_SCAN = os.environ.get("DLI_BLOCK_SCAN", "1") != "0"             # A/B knob: block-parallel lightning prefill
 PREFILL_TILE_TOKENS = 64                                                # queries per prefill tile of these stacks
 
@@ -198,6 +199,12 @@ def token_attention(out: torch.Tensor, q1: torch.Tensor, q2: Optional[torch.Tens
                                      meta.prefill_tile_seq, meta.prefill_tile_q0, meta.num_prefill_tiles,
                                      meta.counts if meta.counts_on_device else None, G, Dv, scale, window, temp, r1, r2):
                 rows = meta.num_decode
+        T, H = q1.shape[0], q1.shape[1]
+        todo = T if rows < 0 else rows                       # tokens the tile kernel left (all of them in a pure decode step)
+        if (HEAD_DECODE and todo > 0 and q1.dtype == torch.bfloat16 and H // G >= 8 and meta.num_prefill_tiles == (0 if rows < 0 else meta.num_prefill_tiles)
+                and lib.sm_head_decode_attention(out, q1, q2, k_cache, v_cache, meta.block_tables, meta.positions, meta.token_seq,
+                                                 G, Dv, scale, window, temp, r1, r2, todo)):
+            rows = 0                                         # done with the heads as matrix-core columns
         if rows != 0:
             lib.sm_token_attention(out, q1, q2, k_cache, v_cache, meta.block_tables, meta.positions, meta.token_seq,
                                    G, Dv, scale, window, temp, r1, r2, rows)

@@ -159,7 +159,10 @@ def other_size_configs():
     wide["mixer"].update(heads=2, dim=8, rot_dim=8, vdim=8, kv_rank=528, rot={"base": 1000.0, "dims": 8})   # latent wider than 512
     tall = copy.deepcopy(LIGHT)
     tall["mixer"].update(heads=1, dim=264, vdim=8, decay=[0.97])                                                # more than 256 state rows
+    many = copy.deepcopy(LATENT)
+    many["mixer"].update(heads=17, dim=8, rot_dim=8, vdim=16, kv_rank=32, rot={"base": 300.0, "dims": 6})      # two groups of heads
     return {
+        "seventeen latent heads": make_cfg([many, LIGHT], width=64, vocab=77),
         "wide latent, tall state": make_cfg([wide, tall], width=40, vocab=50),
         "square heads, long window": make_cfg([a, l1], width=88, vocab=97, mult=1.0, cap=None),
         "single heads, whole stack three times": make_cfg([a1, m2, l2], width=48, vocab=130, loop=(0, 3, 3), eps=1e-3),

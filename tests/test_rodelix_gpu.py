@@ -49,9 +49,10 @@ def test_first_tokens_and_long_decoding(tmp_path):
     cases.case_first_tokens_and_long_decode(tmp_path, "cuda", "float32")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", sorted(cases.other_size_configs()))
-def test_other_sizes(tmp_path, name):
-    cases.case_other_sizes(tmp_path, "cuda", "float32", name)
+def test_other_sizes(tmp_path, name, dtype):
+    cases.case_other_sizes(tmp_path, "cuda", dtype, name)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
