@@ -29,6 +29,29 @@ template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p =
 template <> __device__ __forceinline__ void stf<uint16_t>(uint16_t* p, float v) { *p = f2bf(v); }
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.f + expf(-x)); }
+// activation of a projection output: for bf16 inputs the hardware exp2 / rcp (relative error ≈ 1e-6, far inside bf16)
+template <typename A> __device__ __forceinline__ float silu_act(float x);
+template <> __device__ __forceinline__ float silu_act<float>(float x) { return silu_f(x); }
+template <> __device__ __forceinline__ float silu_act<uint16_t>(float x) {
+  return x * fast_rcp(1.f + fast_exp2(-1.4426950408889634f * x));
+}
+
+// 4 consecutive row elements ↔ fp32 (16-byte / 8-byte accesses; the callers check divisibility and alignment)
+template <typename A> __device__ __forceinline__ f32x4 ld4(const A* p);
+template <> __device__ __forceinline__ f32x4 ld4<float>(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+template <> __device__ __forceinline__ f32x4 ld4<uint16_t>(const uint16_t* p) {
+  const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+  return f32x4{bf2f((uint16_t)v[0]), bf2f((uint16_t)v[1]), bf2f((uint16_t)v[2]), bf2f((uint16_t)v[3])};
+}
+template <typename A> __device__ __forceinline__ void st4(A* p, f32x4 v);
+template <> __device__ __forceinline__ void st4<float>(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+template <> __device__ __forceinline__ void st4<uint16_t>(uint16_t* p, f32x4 v) {
+  bf16x4 o;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) o[j] = (short)f2bf(v[j]);
+  *reinterpret_cast<bf16x4*>(p) = o;
+}
+__device__ __forceinline__ bool aligned_to(const void* p, int bytes) { return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) == 0; }
 
 // q (fp32, LDS) · one cache row: 16-byte loads where the row allows them
 template <typename A> __device__ __forceinline__ float dot_row(const float* __restrict__ qs, const A* __restrict__ kr, int n);
@@ -60,13 +83,29 @@ template <> __device__ __forceinline__ float dot_row<uint16_t>(const float* __re
 
 // mean and 1/sqrt(var + eps) of a row held in LDS (two passes: the variance is the mean squared deviation)
 __device__ __forceinline__ void row_stats(const float* row, int W, float eps, float* red, float& mean, float& inv) {
+  const bool v4 = (W & 3) == 0;
   float s = 0.f;
-  for (int i = threadIdx.x; i < W; i += NT) s += row[i];
+  if (v4) {
+    for (int i = threadIdx.x * 4; i < W; i += NT * 4) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(row + i);
+      s += (a[0] + a[1]) + (a[2] + a[3]);
+    }
+  } else {
+    for (int i = threadIdx.x; i < W; i += NT) s += row[i];
+  }
   mean = block_sum<NT>(s, red) / (float)W;
   float v = 0.f;
-  for (int i = threadIdx.x; i < W; i += NT) {
-    const float d = row[i] - mean;
-    v += d * d;
+  if (v4) {
+    for (int i = threadIdx.x * 4; i < W; i += NT * 4) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(row + i);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v += (a[j] - mean) * (a[j] - mean);
+    }
+  } else {
+    for (int i = threadIdx.x; i < W; i += NT) {
+      const float d = row[i] - mean;
+      v += d * d;
+    }
   }
   inv = 1.f / sqrtf(block_sum<NT>(v, red) / (float)W + eps);
 }
@@ -78,11 +117,26 @@ __global__ __launch_bounds__(NT) void layer_norm_kernel(const float* __restrict_
   extern __shared__ float sh[];
   __shared__ float red[NT / 64];
   const int64_t t = blockIdx.x;
-  for (int i = threadIdx.x; i < W; i += NT) sh[i] = x[t * W + i];
+  const bool v4 = (W & 3) == 0;
+  if (v4) {
+    for (int i = threadIdx.x * 4; i < W; i += NT * 4) *reinterpret_cast<f32x4*>(sh + i) = ld4<float>(x + t * W + i);
+  } else {
+    for (int i = threadIdx.x; i < W; i += NT) sh[i] = x[t * W + i];
+  }
   __syncthreads();
   float mean, inv;
   row_stats(sh, W, eps, red, mean, inv);
-  for (int i = threadIdx.x; i < W; i += NT) stf<O>(out + t * W + i, (sh[i] - mean) * inv * w[i] + b[i]);
+  if (v4) {
+    for (int i = threadIdx.x * 4; i < W; i += NT * 4) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(sh + i), ww = ld4<float>(w + i), bb = ld4<float>(b + i);
+      f32x4 o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = (a[j] - mean) * inv * ww[j] + bb[j];
+      st4<O>(out + t * W + i, o);
+    }
+  } else {
+    for (int i = threadIdx.x; i < W; i += NT) stf<O>(out + t * W + i, (sh[i] - mean) * inv * w[i] + b[i]);
+  }
 }
 
 // h[t] = g[t] + (g[t-1] - g[t]) * mix with g = layer_norm(x (+ add)); g[t-1] is recomputed from the row above inside a
@@ -106,25 +160,66 @@ __global__ __launch_bounds__(NT) void ln_shift_kernel(const float* __restrict__ 
   const int mode = pos == 0 ? 0 : (first ? (slot >= 0 ? 1 : 0) : 2);
   float* cur = sh;
   float* prv = sh + W;
-  for (int i = threadIdx.x; i < W; i += NT) {
-    float v = x[t * W + i];
-    if (add != nullptr) {
-      v += add[t * W + i];
-      xout[t * W + i] = v;
+  const bool v4 = (W & 3) == 0;
+  if (v4) {
+    for (int i = threadIdx.x * 4; i < W; i += NT * 4) {
+      f32x4 v = ld4<float>(x + t * W + i);
+      if (add != nullptr) {
+        const f32x4 a = ld4<float>(add + t * W + i);
+        v = f32x4{v[0] + a[0], v[1] + a[1], v[2] + a[2], v[3] + a[3]};
+        st4<float>(xout + t * W + i, v);
+      }
+      *reinterpret_cast<f32x4*>(cur + i) = v;
+      if (mode == 2) {
+        f32x4 u = ld4<float>(x + (t - 1) * W + i);
+        if (add != nullptr) {
+          const f32x4 a = ld4<float>(add + (t - 1) * W + i);
+          u = f32x4{u[0] + a[0], u[1] + a[1], u[2] + a[2], u[3] + a[3]};
+        }
+        *reinterpret_cast<f32x4*>(prv + i) = u;
+      }
     }
-    cur[i] = v;
-    if (mode == 2) prv[i] = x[(t - 1) * W + i] + (add != nullptr ? add[(t - 1) * W + i] : 0.f);
+  } else {
+    for (int i = threadIdx.x; i < W; i += NT) {
+      float v = x[t * W + i];
+      if (add != nullptr) {
+        v += add[t * W + i];
+        xout[t * W + i] = v;
+      }
+      cur[i] = v;
+      if (mode == 2) prv[i] = x[(t - 1) * W + i] + (add != nullptr ? add[(t - 1) * W + i] : 0.f);
+    }
   }
   __syncthreads();
   float mean, inv, pmean = 0.f, pinv = 0.f;
   row_stats(cur, W, eps, red, mean, inv);
   if (mode == 2) row_stats(prv, W, eps, red, pmean, pinv);
-  for (int i = threadIdx.x; i < W; i += NT) {
-    const float g = (cur[i] - mean) * inv * w[i] + b[i];
-    float p = 0.f;
-    if (mode == 1) p = state[(int64_t)slot * W + i];
-    else if (mode == 2) p = (prv[i] - pmean) * pinv * w[i] + b[i];
-    stf<O>(out + t * W + i, g + (p - g) * mix[i]);
+  if (v4) {
+    for (int i = threadIdx.x * 4; i < W; i += NT * 4) {
+      const f32x4 c4 = *reinterpret_cast<const f32x4*>(cur + i), ww = ld4<float>(w + i), bb = ld4<float>(b + i), mm = ld4<float>(mix + i);
+      f32x4 p4 = {0.f, 0.f, 0.f, 0.f};
+      if (mode == 1) p4 = ld4<float>(state + (int64_t)slot * W + i);
+      else if (mode == 2) {
+        const f32x4 u = *reinterpret_cast<const f32x4*>(prv + i);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) p4[j] = (u[j] - pmean) * pinv * ww[j] + bb[j];
+      }
+      f32x4 o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float g = (c4[j] - mean) * inv * ww[j] + bb[j];
+        o[j] = g + (p4[j] - g) * mm[j];
+      }
+      st4<O>(out + t * W + i, o);
+    }
+  } else {
+    for (int i = threadIdx.x; i < W; i += NT) {
+      const float g = (cur[i] - mean) * inv * w[i] + b[i];
+      float p = 0.f;
+      if (mode == 1) p = state[(int64_t)slot * W + i];
+      else if (mode == 2) p = (prv[i] - pmean) * pinv * w[i] + b[i];
+      stf<O>(out + t * W + i, g + (p - g) * mix[i]);
+    }
   }
 }
 
@@ -158,19 +253,45 @@ __global__ __launch_bounds__(NT) void add_ln_kernel(float* __restrict__ x, const
   extern __shared__ float sh[];
   __shared__ float red[NT / 64];
   const int64_t t = blockIdx.x;
-  for (int i = threadIdx.x; i < W; i += NT) sh[i] = ldf<Y>(y + t * y_stride + i);
+  const bool v4 = (W & 3) == 0 && (y_stride & 3) == 0 && aligned_to(y, 4 * sizeof(Y));
+  if (v4) {
+    for (int i = threadIdx.x * 4; i < W; i += NT * 4) *reinterpret_cast<f32x4*>(sh + i) = ld4<Y>(y + t * y_stride + i);
+  } else {
+    for (int i = threadIdx.x; i < W; i += NT) sh[i] = ldf<Y>(y + t * y_stride + i);
+  }
   __syncthreads();
   float mean, inv;
   row_stats(sh, W, eps, red, mean, inv);
-  for (int i = threadIdx.x; i < W; i += NT) {
-    const float v = x[t * W + i] + mult * ((sh[i] - mean) * inv * w1[i] + b1[i]);
-    x[t * W + i] = v;
-    sh[i] = v;
+  if (v4) {
+    for (int i = threadIdx.x * 4; i < W; i += NT * 4) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(sh + i), ww = ld4<float>(w1 + i), bb = ld4<float>(b1 + i);
+      f32x4 v = ld4<float>(x + t * W + i);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] += mult * ((a[j] - mean) * inv * ww[j] + bb[j]);
+      st4<float>(x + t * W + i, v);
+      *reinterpret_cast<f32x4*>(sh + i) = v;
+    }
+  } else {
+    for (int i = threadIdx.x; i < W; i += NT) {
+      const float v = x[t * W + i] + mult * ((sh[i] - mean) * inv * w1[i] + b1[i]);
+      x[t * W + i] = v;
+      sh[i] = v;
+    }
   }
   if (w2 == nullptr) return;
   __syncthreads();
   row_stats(sh, W, eps, red, mean, inv);
-  for (int i = threadIdx.x; i < W; i += NT) stf<O>(out + t * W + i, (sh[i] - mean) * inv * w2[i] + b2[i]);
+  if (v4) {
+    for (int i = threadIdx.x * 4; i < W; i += NT * 4) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(sh + i), ww = ld4<float>(w2 + i), bb = ld4<float>(b2 + i);
+      f32x4 o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = (a[j] - mean) * inv * ww[j] + bb[j];
+      st4<O>(out + t * W + i, o);
+    }
+  } else {
+    for (int i = threadIdx.x; i < W; i += NT) stf<O>(out + t * W + i, (sh[i] - mean) * inv * w2[i] + b2[i]);
+  }
 }
 
 // o: `parts` planes of partial sums [parts][T][N] (the scan cuts the state rows into parts); the row is their sum
@@ -543,30 +664,33 @@ __global__ __launch_bounds__(NT) void token_attention_kernel(
   }
 }
 
-// combine the nsplit partial results of a (token, head): part [T][H][nsplit][2 + Dv] = (max, sum, unnormalised output)
+// combine the nsplit (≤ 16) partial results of a (token, head): part [T][H][nsplit][2 + Dv] = (max, sum, unnormalised output)
 template <typename A>
-__global__ __launch_bounds__(64) void token_attention_merge_kernel(A* __restrict__ out, int64_t o_ts, int64_t o_hs,
-                                                                   const float* __restrict__ part,
-                                                                   const int* __restrict__ token_seq, int H, int Dv,
-                                                                   int nsplit) {
+__global__ __launch_bounds__(128) void token_attention_merge_kernel(A* __restrict__ out, int64_t o_ts, int64_t o_hs,
+                                                                    const float* __restrict__ part,
+                                                                    const int* __restrict__ token_seq, int H, int Dv,
+                                                                    int nsplit) {
   const int64_t t = blockIdx.x;
   const int h = blockIdx.y;
   if (token_seq[t] < 0) return;
   const float* pr = part + (t * H + h) * nsplit * (int64_t)(Dv + 2);
   float M = -INFINITY;
   for (int z = 0; z < nsplit; ++z) M = fmaxf(M, pr[z * (Dv + 2)]);
+  float f[16];
   float L = 0.f;
-  for (int z = 0; z < nsplit; ++z) {
-    const float mz = pr[z * (Dv + 2)];
-    if (mz != -INFINITY) L += expf(mz - M) * pr[z * (Dv + 2) + 1];
+#pragma unroll
+  for (int z = 0; z < 16; ++z) {
+    const float mz = z < nsplit ? pr[z * (Dv + 2)] : -INFINITY;
+    f[z] = mz == -INFINITY ? 0.f : expf(mz - M);
+    if (z < nsplit) L += f[z] * pr[z * (Dv + 2) + 1];
   }
-  for (int e = threadIdx.x; e < Dv; e += 64) {
+  const float rl = 1.f / L;
+  for (int e = threadIdx.x; e < Dv; e += 128) {
     float o = 0.f;
-    for (int z = 0; z < nsplit; ++z) {
-      const float mz = pr[z * (Dv + 2)];
-      if (mz != -INFINITY) o += expf(mz - M) * pr[z * (Dv + 2) + 2 + e];
-    }
-    stf<A>(out + t * o_ts + h * o_hs + e, o / L);
+#pragma unroll
+    for (int z = 0; z < 16; ++z)
+      if (z < nsplit) o += f[z] * pr[z * (Dv + 2) + 2 + e];
+    stf<A>(out + t * o_ts + h * o_hs + e, o * rl);
   }
 }
 
@@ -977,11 +1101,11 @@ __global__ __launch_bounds__(64) void lightning_scan_kernel(const A* __restrict_
     for (int r = 0; r < PER; ++r) {
       const int i = lane + 64 * r;
       if (i < DMAX) {
-        if (MODE != 1) qs[buf][i] = silu_f(nq[r]);
-        ks[buf][i] = silu_f(nk[r]);
+        if (MODE != 1) qs[buf][i] = silu_act<A>(nq[r]);
+        ks[buf][i] = silu_act<A>(nk[r]);
       }
     }
-    const float ve = silu_f(nv);
+    const float ve = silu_act<A>(nv);
     if (t + 1 < t1) fetch(t + 1);
     __syncthreads();                       // one wave: publishes qs / ks of this token (the other buffer is being refilled next trip)
     float o = 0.f;
@@ -1166,7 +1290,7 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
   else SM_ATT_V(8);
 #undef SM_ATT_V
   if (nsplit > 1)
-    SM_DISPATCH_BF16(bf16, A, hipLaunchKernelGGL(token_attention_merge_kernel<A>, dim3(rows, H), dim3(64), 0, stream, (A*)out, o_ts,
+    SM_DISPATCH_BF16(bf16, A, hipLaunchKernelGGL(token_attention_merge_kernel<A>, dim3(rows, H), dim3(128), 0, stream, (A*)out, o_ts,
                                                  o_hs, (const float*)part, token_seq, H, Dv, nsplit));
 }
 
@@ -1257,7 +1381,7 @@ bool launch_sm_head_decode_attention(void* out, int64_t o_ts, int64_t o_hs, cons
   else SM_HD(18, 8);
 #undef SM_HD
   if (nsplit > 1)
-    hipLaunchKernelGGL(token_attention_merge_kernel<uint16_t>, dim3(rows, H), dim3(64), 0, stream, (uint16_t*)out, o_ts, o_hs,
+    hipLaunchKernelGGL(token_attention_merge_kernel<uint16_t>, dim3(rows, H), dim3(128), 0, stream, (uint16_t*)out, o_ts, o_hs,
                        (const float*)part, token_seq, H, Dv, nsplit);
   return true;
 }
@@ -1266,7 +1390,7 @@ bool launch_sm_head_decode_attention(void* out, int64_t o_ts, int64_t o_hs, cons
 int sm_head_decode_splits(int rows, int H, int G) {
   const int per = H / G;
   const int wgs = std::max(rows * G * ((per + 15) / 16), 1);
-  return std::max(1, std::min(16, 512 / wgs));
+  return std::max(1, std::min(8, 512 / wgs));
 }
 
 // rows of the state one wave keeps: D is cut into parts so that a wave's per-token loop is short and more waves share the work

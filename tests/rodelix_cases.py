@@ -166,7 +166,7 @@ def other_size_configs():
         "wide latent, tall state": make_cfg([wide, tall], width=40, vocab=50),
         "square heads, long window": make_cfg([a, l1], width=88, vocab=97, mult=1.0, cap=None),
         "single heads, whole stack three times": make_cfg([a1, m2, l2], width=48, vocab=130, loop=(0, 3, 3), eps=1e-3),
-        "loop at the end": make_cfg([m1, l2, a], width=56, vocab=64, loop=(2, 3, 2), mult=0.1, cap=3.0),
+        "loop at the end": make_cfg([m1, l2, a], width=54, vocab=64, loop=(2, 3, 2), mult=0.1, cap=3.0),
     }
 
 
