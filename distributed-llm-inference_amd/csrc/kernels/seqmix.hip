@@ -773,6 +773,7 @@ __global__ __launch_bounds__(NT * HW) void tile_attention_kernel(
   for (int i = 0; i < MTMAX; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int kchunks = Dk >> 3, vchunks = Dv >> 3;
+  const bool vfromk = vc == kc && rowv == rowk && vhead == Dk;     // latent attention: one row is key and value
   for (int kb = kb_lo; kb <= kb_hi; ++kb) {
     __syncthreads();                                      // everyone is done with the previous page
     const int64_t page_row = (int64_t)bt[kb] * kBlockTokens;
@@ -781,9 +782,11 @@ __global__ __launch_bounds__(NT * HW) void tile_attention_kernel(
       *reinterpret_cast<bf16x8*>(Ks + row * KST + 8 * ch) =
           *reinterpret_cast<const bf16x8*>(kc + (page_row + row) * rowk + g * Dk + 8 * ch);
     }
+    if (vfromk) __syncthreads();                          // values = leading columns of the key rows just staged
     for (int i = threadIdx.x; i < 32 * vchunks; i += TNT) {
       const int row = i & 31, ch = i >> 5;
-      const bf16x8 v = *reinterpret_cast<const bf16x8*>(vc + (page_row + row) * rowv + g * vhead + 8 * ch);
+      const bf16x8 v = vfromk ? *reinterpret_cast<const bf16x8*>(Ks + row * KST + 8 * ch)
+                              : *reinterpret_cast<const bf16x8*>(vc + (page_row + row) * rowv + g * vhead + 8 * ch);
       const int slot = ((row & 15) >> 2) * 8 + (row >> 4) * 4 + (row & 3);
 #pragma unroll
       for (int j = 0; j < 8; ++j) Vt[(8 * ch + j) * VST + slot] = (uint16_t)v[j];
@@ -921,6 +924,7 @@ __global__ __launch_bounds__(NT) void head_decode_attention_kernel(
 #pragma unroll
   for (int i = 0; i < MTQ; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int kchunks = Dk >> 3, vchunks = Dv >> 3;
+  const bool vfromk = vc == kc && rowv == rowk && vhead == Dk;     // latent attention: one row is key and value
   for (int kb = kb_begin; kb <= kb_end; ++kb) {
     __syncthreads();
     const int64_t page_row = (int64_t)bt[kb] * kBlockTokens;
@@ -929,9 +933,11 @@ __global__ __launch_bounds__(NT) void head_decode_attention_kernel(
       *reinterpret_cast<bf16x8*>(Ks + row * KST + 8 * ch) =
           *reinterpret_cast<const bf16x8*>(kc + (page_row + row) * rowk + g * Dk + 8 * ch);
     }
+    if (vfromk) __syncthreads();                          // values = leading columns of the key rows just staged
     for (int i = threadIdx.x; i < 32 * vchunks; i += NT) {
       const int row = i & 31, ch = i >> 5;
-      const bf16x8 v = *reinterpret_cast<const bf16x8*>(vc + (page_row + row) * rowv + g * vhead + 8 * ch);
+      const bf16x8 v = vfromk ? *reinterpret_cast<const bf16x8*>(Ks + row * KST + 8 * ch)
+                              : *reinterpret_cast<const bf16x8*>(vc + (page_row + row) * rowv + g * vhead + 8 * ch);
       const int slot = ((row & 15) >> 2) * 8 + (row >> 4) * 4 + (row & 3);
 #pragma unroll
       for (int j = 0; j < 8; ++j) Vt[(8 * ch + j) * VST + slot] = (uint16_t)v[j];

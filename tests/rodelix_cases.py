@@ -90,8 +90,9 @@ def _peaky(Wt):
             Wt[k] = Wt[k] * 0.05
 
 
-def case_window_edges(tmp, device, dtype):
+def case_window_edges(tmp, device, dtype, heads=4, kv_heads=2):
     layer = copy.deepcopy(ATTN)
+    layer["mixer"].update(heads=heads, kv_heads=kv_heads)
     layer["mixer"]["mask"]["size"] = 33                       # crosses a 32-token page by one
     cfg = make_cfg([layer, layer], width=64)
     W, rig = _setup(tmp, cfg, dtype, device, seed=11, edit=_peaky)
@@ -102,7 +103,7 @@ def case_window_edges(tmp, device, dtype):
         other = copy.deepcopy(cfg)
         for l in other["layers"]:
             l["mixer"]["mask"]["size"] += off
-        assert rel_err(expect(other, W, toks)[40:], want[40:]) > 20 * TOL[dtype]
+        assert rel_err(expect(other, W, toks)[40:], want[40:]) > 5 * TOL[dtype]
     got = rig.run({"p": toks}, alone("p", 120, [120]))["p"]
     _check(got, want, dtype, "window in a prompt")
     got = rig.run({"d": toks}, alone("d", 120, [30, 1, 1, 1, 1, 1, 1, 2, 31] + [1] * 60))["d"]
@@ -119,7 +120,7 @@ def case_far_key(tmp, device, dtype):
     want = expect(cfg, W, toks)
     changed = list(toks)
     changed[1] = (toks[1] + 17) % cfg["vocab"]
-    assert rel_err(expect(cfg, W, changed)[-20:], want[-20:]) > 20 * TOL[dtype]      # position 1 reaches the last rows
+    assert rel_err(expect(cfg, W, changed)[-20:], want[-20:]) > 5 * TOL[dtype]       # position 1 reaches the last rows
     got = rig.run({"p": toks}, alone("p", 330, [300] + [1] * 30))["p"]
     _check(got, want, dtype, "far keys, prompt then decoding")
     got = rig.run({"c": toks}, alone("c", 330, [64, 63, 2, 129]))["c"]
@@ -161,7 +162,12 @@ def other_size_configs():
     tall["mixer"].update(heads=1, dim=264, vdim=8, decay=[0.97])                                                # more than 256 state rows
     many = copy.deepcopy(LATENT)
     many["mixer"].update(heads=17, dim=8, rot_dim=8, vdim=16, kv_rank=32, rot={"base": 300.0, "dims": 6})      # two groups of heads
+    fan = copy.deepcopy(ATTN)
+    fan["mixer"].update(heads=8, kv_heads=1, dim=16, vdim=32, mask={"size": 45})                                  # eight query heads on one key head
+    fan2 = copy.deepcopy(ATTN)
+    fan2["mixer"].update(heads=24, kv_heads=2, dim=8, vdim=16, mask={"size": 9})
     return {
+        "many query heads per key head": make_cfg([fan, fan2], width=64, vocab=90, loop=(0, 1, 2)),
         "seventeen latent heads": make_cfg([many, LIGHT], width=64, vocab=77),
         "wide latent, tall state": make_cfg([wide, tall], width=40, vocab=50),
         "square heads, long window": make_cfg([a, l1], width=88, vocab=97, mult=1.0, cap=None),

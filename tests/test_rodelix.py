@@ -27,12 +27,15 @@ def test_pages_and_slots_used_again(tmp_path):
     cases.case_reuse(tmp_path, "cpu", "float32")
 
 
-def test_window_edges(tmp_path):
-    cases.case_window_edges(tmp_path, "cpu", "float32")
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("heads,kv_heads", [(4, 2), (8, 1)])
+def test_window_edges(tmp_path, heads, kv_heads, dtype):
+    cases.case_window_edges(tmp_path, "cpu", dtype, heads, kv_heads)
 
 
 def test_far_keys(tmp_path):
     cases.case_far_key(tmp_path, "cpu", "float32")
+
 
 
 def test_first_tokens_and_long_decoding(tmp_path):

@@ -37,8 +37,10 @@ def test_pages_and_slots_used_again(tmp_path, dtype):
     cases.case_reuse(tmp_path, "cuda", dtype)
 
 
-def test_window_edges(tmp_path):
-    cases.case_window_edges(tmp_path, "cuda", "float32")
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads", [(4, 2), (8, 1)])           # (8, 1): decode rows take the heads-as-columns kernel
+def test_window_edges(tmp_path, heads, kv_heads, dtype):
+    cases.case_window_edges(tmp_path, "cuda", dtype, heads, kv_heads)
 
 
 def test_far_keys(tmp_path):
