@@ -46,11 +46,11 @@ def _headers():
     return out
 
 
-def build_runtime(verbose: bool = False) -> str:
+def build_runtime(verbose: bool = False, force: bool = False) -> str:
     import pybind11
 
     src = os.path.join(CSRC, "runtime", "block_manager.cpp")
-    if _newer([src, os.path.join(CSRC, "runtime", "block_manager.h")], RUNTIME_SO):
+    if force or _newer([src, os.path.join(CSRC, "runtime", "block_manager.h")], RUNTIME_SO):
         cxx = os.environ.get("CXX", "g++")
         # several processes may get here at once on a fresh checkout (TP workers, router replicas import the module
         # concurrently): each links into its own temp file and renames it into place — nobody can import a half-written .so
@@ -81,7 +81,7 @@ def _torch_flags():
     return inc, defs, libs
 
 
-def build_kernels(verbose: bool = False) -> str:
+def build_kernels(verbose: bool = False, force: bool = False) -> str:
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     kdir = os.path.join(CSRC, "kernels")
     os.makedirs(OBJ_DIR, exist_ok=True)
@@ -98,11 +98,11 @@ def build_kernels(verbose: bool = False) -> str:
     for src in kernel_srcs:
         obj = os.path.join(OBJ_DIR, os.path.basename(src) + ".o")
         objs.append(obj)
-        if _newer([src] + hdrs, obj):
+        if force or _newer([src] + hdrs, obj):
             jobs.append([hipcc] + common + ["-c", src, "-o", obj])
     bobj = os.path.join(OBJ_DIR, "torch_bindings.o")
     objs.append(bobj)
-    if _newer([binding_src] + hdrs, bobj):
+    if force or _newer([binding_src] + hdrs, bobj):
         jobs.append([hipcc] + common + inc + defs + ["-x", "hip", "-c", binding_src, "-o", bobj])
 
     def one(cmd):
@@ -124,10 +124,11 @@ def build_kernels(verbose: bool = False) -> str:
     return KERNELS_SO
 
 
-def build_all(verbose: bool = False):
-    return build_runtime(verbose), build_kernels(verbose)
+def build_all(verbose: bool = False, force: bool = False):
+    """``force``: compile every translation unit again, whatever is already built (the "does it build" check)."""
+    return build_runtime(verbose, force), build_kernels(verbose, force)
 
 
 if __name__ == "__main__":
-    for path in build_all(verbose="-q" not in sys.argv):
+    for path in build_all(verbose="-q" not in sys.argv, force="--force" in sys.argv):
         print("built", path)
