@@ -20,7 +20,13 @@ class MixerSpec:
 
     ``kind``: ``"attention"`` (grouped-query softmax attention over a sliding window, unit-RMS queries / keys, per-head
     temperature and logarithmic distance penalty), ``"latent_attention"`` (keys / values expanded from a cached low-rank
-    latent + one shared rotated key part) or ``"lightning"`` (linear attention with a per-head decay and a recurrent state)."""
+    latent + one shared rotated key part), ``"lightning"`` (linear attention with a per-head decay and a recurrent state),
+    ``"sink_attention"`` (causal grouped-query attention: q / k normalised over the whole projection, half-split rotation of
+    the leading ``rot_dims`` entries of every head with optionally stretched frequencies, a per-head sink in the softmax
+    denominator, softmax weights mixed across heads, sigmoid output gate), ``"time_mix"`` (recurrence with a per-token,
+    per-channel decay from a low-rank projection, a bonus for the current token and a ``[D, D]`` state per head; all five
+    projections read their own blend of the token's and the previous token's input) or ``"parallel"`` (the mixers in
+    ``parts`` read the same input; their outputs are summed with the weights ``part_scales``)."""
     kind: str
     heads: int
     dim: int                            # per-head query / key size (latent attention: the unrotated part)
@@ -33,26 +39,38 @@ class MixerSpec:
     rot_base: float = 10000.0
     rot_dims: int = 0                   # leading entries of the rotated part that are actually rotated
     decay: tuple = ()                   # lightning: per-head state decay
-    ff: int = 0                         # feed-forward inner width (0: the layer has none)
-    ff_kind: str = "dense"
+    rot_scaling: tuple = ()             # sink attention: (factor, original length, fast turns, slow turns) or ()
+    lora: int = 0                       # time mix: rank of the decay projection
+    parts: tuple = ()                   # parallel: the mixers run side by side (MixerSpec each)
+    part_scales: tuple = ()             # parallel: weight of every part's output
+    ff: int = 0                         # feed-forward inner width (0: the layer has none); routed: of ONE expert
+    ff_kind: str = "dense"              # "dense" | "moe" (sigmoid-routed squared-ReLU experts + optional gated shared expert)
+    experts: int = 0                    # moe: number of routed experts
+    top: int = 0                        # moe: experts per token
+    router_scale: float = 1.0           # moe: multiplies the chosen experts' scores
+    shared_ff: int = 0                  # moe: inner width of the expert every token takes (0: none)
 
     @property
     def stateful(self) -> bool:
-        return self.kind == "lightning"
+        return self.kind in ("lightning", "time_mix") or any(p.stateful for p in self.parts)
 
     @property
     def cache_row(self) -> tuple:
         """Widths of the per-token rows this mixer keeps in the paged cache: ``(key row, value row)``; a latent mixer keeps
         one row (latent | rotated key) that serves as both; a recurrent one keeps none."""
-        if self.kind == "attention":
+        if self.kind in ("attention", "sink_attention"):
             return self.kv_heads * self.dim, self.kv_heads * self.vdim
+        if self.kind == "parallel":
+            return tuple(sum(w) for w in zip(*(p.cache_row for p in self.parts)))
         if self.kind == "latent_attention":
             return self.kv_rank + self.rot_dim, 0
         return 0, 0
 
     @property
     def state_shape(self) -> tuple:
-        return (self.heads, self.dim, self.vdim) if self.kind == "lightning" else ()
+        if self.kind == "parallel":
+            return next((p.state_shape for p in self.parts if p.state_shape), ())
+        return (self.heads, self.dim, self.vdim) if self.kind in ("lightning", "time_mix") else ()
 
 
 @dataclass
@@ -112,6 +130,9 @@ class ModelConfig:
         if self.layer_specs:
             tot = 2 * v * h + 2 * h
             for m in self.layer_specs:
+                if m.kind == "parallel":
+                    tot += _parallel_layer_params(m, h)
+                    continue
                 tot += 9 * h + 2 * h * m.ff
                 if m.kind == "attention":
                     tot += h * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) + m.heads * m.vdim * h
@@ -128,6 +149,21 @@ class ModelConfig:
             mlp = 3 * h * i * max(self.num_experts, 1)
         emb = v * h * (1 if self.tie_embeddings else 2)
         return l * (attn + mlp) + emb
+
+
+def _parallel_layer_params(m: MixerSpec, h: int) -> int:
+    """Parameters of one gated parallel layer (two scalar norms, residual gates, the side-by-side mixers, routed FFN)."""
+    tot = 2 + 2 * (h * h + h) if m.ff else 1 + h * h + h
+    for p in m.parts:
+        if p.kind == "sink_attention":
+            tot += h * (2 * p.heads * p.dim + p.kv_heads * (p.dim + p.vdim)) + 2 * p.heads * p.vdim * h \
+                + (p.heads + p.kv_heads) * p.dim + p.heads * p.heads + p.heads
+        else:
+            c = p.heads * p.dim
+            tot += 5 * h + 5 * c * h + p.lora * (h + c) + 3 * c
+    if m.ff:
+        tot += m.experts * (2 * h * m.ff + h) + (2 * h * m.shared_ff + h if m.shared_ff else 0)
+    return tot
 
 
 def _rodelix_spec(entry: dict) -> MixerSpec:
@@ -162,7 +198,62 @@ def rodelix_config(cfg: dict, name: str = "rodelix", dtype: str = "bfloat16") ->
                        residual_mult=float(cfg.get("residual_mult", 1.0)), logit_softcap=float(cfg.get("logit_softcap") or 0.0))
 
 
-_CONFIG_READERS = {"Rodelix": rodelix_config}
+def _vibunex_spec(entry: dict, index: int, shapes: Optional[dict]) -> MixerSpec:
+    if entry["type"] != "parallel":
+        raise ValueError(f"unknown layer type {entry['type']!r}")
+    m, mlp = entry["mixer"], entry.get("mlp")
+    a, b = m["left"], m["right"]
+    rot = a.get("rot") or {}
+    sc = rot.get("scaling")
+    left = MixerSpec(kind="sink_attention", heads=int(a["heads"]), kv_heads=int(a["kv_heads"]), dim=int(a["dim"]),
+                     vdim=int(a["vdim"]), scale=float(a["scale"]), rot_base=float(rot.get("base", 10000.0)),
+                     rot_dims=int(rot.get("dims", 0)),
+                     rot_scaling=(float(sc["factor"]), float(sc["original"]), float(sc["fast"]), float(sc["slow"])) if sc else ())
+    # the rank of the decay projection is a tensor's shape, not a configuration entry
+    lora = b.get("lora") or (shapes or {}).get(f"l{index}.mix.right.w1", (0,))[0]
+    if not lora:
+        raise ValueError(f"layer {index}: the decay projection's rank is neither in the configuration nor a checkpoint tensor's shape")
+    right = MixerSpec(kind="time_mix", heads=int(b["heads"]), dim=int(b["dim"]), vdim=int(b["dim"]), lora=int(lora))
+    ff = {}
+    if mlp:
+        if mlp.get("kind", "moe") != "moe":
+            raise ValueError(f"unknown feed-forward kind {mlp.get('kind')!r}")
+        r, sh = mlp["router"], mlp.get("shared")
+        ff = dict(ff=int(mlp["expert"]["ff"]), ff_kind="moe", experts=int(r["experts"]), top=int(r["top"]),
+                  router_scale=float(r.get("scale", 1.0)), shared_ff=int(sh["ff"]) if sh else 0)
+    return MixerSpec(kind="parallel", heads=left.heads, dim=left.dim, vdim=left.vdim, kv_heads=left.kv_heads, parts=(left, right),
+                     part_scales=(float(m.get("left_scale", 1.0)), float(m.get("right_scale", 1.0))), **ff)
+
+
+def vibunex_config(cfg: dict, name: str = "vibunex", dtype: str = "bfloat16", shapes: Optional[dict] = None) -> ModelConfig:
+    """``ModelConfig`` of a Vibunex checkpoint from the dict its ``config.json`` holds (``shapes``: tensor name → shape of
+    the checkpoint, for the sizes the configuration leaves to the tensors)."""
+    specs = tuple(_vibunex_spec(e, i, shapes) for i, e in enumerate(cfg["layers"]))
+    left = specs[0].parts[0]
+    return ModelConfig(name=name, arch="vibunex", vocab_size=int(cfg["vocab"]), hidden_size=int(cfg["width"]),
+                       intermediate_size=max(max(s.ff, s.shared_ff) for s in specs), num_layers=len(specs), num_heads=left.heads,
+                       num_kv_heads=left.kv_heads, head_dim=left.dim, max_position=1 << 24, rms_eps=float(cfg["norm"]["eps"]),
+                       dtype=dtype, bos_token_id=0, eos_token_id=-1, layer_specs=specs,
+                       residual_mult=float(cfg.get("residual_mult", 1.0)))
+
+
+_CONFIG_READERS = {"Rodelix": rodelix_config, "Vibunex": vibunex_config}
+
+
+def safetensors_shapes(path: str) -> dict:
+    """Tensor name → shape of every ``*.safetensors`` file under ``path`` (headers only: 8-byte length + JSON)."""
+    import glob
+    import json
+    import os
+    import struct
+    out = {}
+    for f in sorted(glob.glob(os.path.join(path, "*.safetensors"))):
+        with open(f, "rb") as fh:
+            (n,) = struct.unpack("<Q", fh.read(8))
+            for k, v in json.loads(fh.read(n)).items():
+                if k != "__metadata__":
+                    out[k] = tuple(v["shape"])
+    return out
 
 
 def load_model_config(path: str, dtype: Optional[str] = None) -> ModelConfig:
@@ -175,6 +266,8 @@ def load_model_config(path: str, dtype: Optional[str] = None) -> ModelConfig:
     if arch not in _CONFIG_READERS:
         raise ValueError(f"no reader for architecture {arch!r} (have {sorted(_CONFIG_READERS)})")
     kw = {"dtype": dtype} if dtype else {}
+    if arch == "Vibunex":
+        kw["shapes"] = safetensors_shapes(path)
     return _CONFIG_READERS[arch](raw, name=os.path.basename(os.path.normpath(path)) or arch.lower(), **kw)
 
 
@@ -246,6 +339,23 @@ MODEL_PRESETS: dict[str, ModelConfig] = {
             {"type": "attention", "mlp": {"kind": "dense", "ff": 128},
              "mixer": {"heads": 2, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": 70}}}]},
         name="tiny-rodelix", dtype="float32"),
+    # gated parallel layers: sink attention beside a decaying recurrence, routed squared-ReLU experts
+    "tiny-vibunex": vibunex_config({
+        "vocab": 320, "width": 96, "residual_mult": 0.5, "norm": {"eps": 1e-5},
+        "layers": [
+            {"type": "parallel",
+             "mixer": {"left_scale": 0.7, "right_scale": 0.8,
+                       "left": {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 16, "scale": 0.2,
+                                "rot": {"base": 10000.0, "dims": 8,
+                                        "scaling": {"factor": 2.0, "original": 64, "fast": 16.0, "slow": 2.0}}},
+                       "right": {"heads": 2, "dim": 24, "lora": 8}},
+             "mlp": {"kind": "moe", "expert": {"ff": 64}, "router": {"experts": 4, "top": 2, "scale": 1.5}, "shared": {"ff": 48}}},
+            {"type": "parallel",
+             "mixer": {"left_scale": 1.0, "right_scale": 0.5,
+                       "left": {"heads": 2, "kv_heads": 2, "dim": 16, "vdim": 32, "scale": 0.25, "rot": {"base": 5000.0, "dims": 16}},
+                       "right": {"heads": 3, "dim": 16, "lora": 4}},
+             "mlp": None}]},
+        name="tiny-vibunex", dtype="float32"),
     "tiny-opt": ModelConfig(name="tiny-opt", arch="opt", vocab_size=512, hidden_size=64,
                             intermediate_size=128, num_layers=2, num_heads=4, num_kv_heads=4,
                             head_dim=16, max_position=512, pos_offset=2, tie_embeddings=True,

@@ -19,8 +19,10 @@ from .layers import random_full_tensor
 from .llama import LlamaForCausalLM
 from .opt import OPTForCausalLM
 from .rodelix import RodelixForCausalLM
+from .vibunex import VibunexForCausalLM
 
-_ARCH = {"llama": LlamaForCausalLM, "mixtral": LlamaForCausalLM, "opt": OPTForCausalLM, "rodelix": RodelixForCausalLM}
+_ARCH = {"llama": LlamaForCausalLM, "mixtral": LlamaForCausalLM, "opt": OPTForCausalLM, "rodelix": RodelixForCausalLM,
+         "vibunex": VibunexForCausalLM}
 
 
 def torch_dtype(name: str) -> torch.dtype:
@@ -54,10 +56,12 @@ def init_random(model, seed: int = 0) -> None:
             w.init_const(0.0)
         elif kind == "half":
             w.init_const(0.5)
+        elif kind == "eye":
+            w.load_full(torch.eye(w.full_shape[0], dtype=torch.float32, device=w.data.device))
         elif kind == "small":                                # per-head constants of order one (kept positive)
             w.load_full(random_full_tensor(name, w.full_shape, torch.float32, w.data.device, seed, 1.0).abs() * 0.5)
-        elif w.data.dim() == 2 and hasattr(model, "checkpoint_sources"):
-            w.init_random(name, seed, std=w.full_shape[1] ** -0.5)   # unit-gain projections: the stack has no trained scale
+        elif w.data.dim() in (2, 3) and hasattr(model, "checkpoint_sources"):
+            w.init_random(name, seed, std=w.full_shape[-1] ** -0.5)  # unit-gain projections: the stack has no trained scale
         else:
             w.init_random(name, seed)
 
@@ -106,7 +110,13 @@ def load_safetensors(model, path: str) -> None:
     for name, w, _kind in model.named_weights():
         if fused is not None:                                # the model names its checkpoint tensors itself
             keys = fused.get(name, [name])
-            full = torch.cat([shards.get(k) for k in keys], dim=0) if len(keys) > 1 else shards.get(keys[0])
+            if isinstance(keys[0], (list, tuple)):                   # stacked: one slice per entry (each a concatenation)
+                full = torch.stack([torch.cat([shards.get(k) for k in ks], dim=0) if len(ks) > 1 else shards.get(ks[0])
+                                    for ks in keys])
+            else:
+                full = torch.cat([shards.get(k) for k in keys], dim=0) if len(keys) > 1 else shards.get(keys[0])
+            if tuple(full.shape) != w.full_shape and full.numel() == w.data.numel():
+                full = full.reshape(w.full_shape)                    # scalars stored 0-d, per-head tables stored [H, D]
         elif ".experts.w" in name:
             full = torch.stack([torch.cat([shards.get(k) for k in ks], dim=0) for ks in _expert_sources(name, cfg)])
         else:

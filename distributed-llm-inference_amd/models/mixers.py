@@ -10,7 +10,17 @@ cache)`` that serves prefill chunks and decode rows of a mixed step alike:
   into the query and the value expansion applied after the softmax, so the cache is all the kernel reads;
 * ``LightningAttention`` – linear attention with a per-head decay: a ``[D, Dv]`` fp32 state per head and sequence.
 
-``MixerLayer`` wraps one of them (and an optional dense feed-forward) in the sandwich
+* ``SinkTalkAttention`` – causal grouped-query attention with whole-projection q / k norm, half-split partial
+  rotation (optionally stretched frequencies), a per-head sink, weights mixed across heads, sigmoid output gate;
+* ``TimeMix`` – recurrence with per-token, per-channel decay (low-rank projection), a bonus for the current token
+  and a ``[D, D]`` fp32 state per head; its five projections read blends of the token's and the previous token's input;
+* ``DualMixer`` – two of the above side by side on the same input, outputs summed with fixed weights.
+
+``RoutedFF`` is a sigmoid-routed mixture of squared-ReLU experts with an optional gated shared expert;
+``GatedParallelLayer`` runs a mixer and a feed-forward on two scalar-gain RMS norms of the same stream and adds
+both, each through a sigmoid gate computed from its own input: ``x += m · (g1 ⊙ mixer(n1) + g2 ⊙ ff(n2))``.
+
+``MixerLayer`` wraps one of the first three (and an optional dense feed-forward) in the sandwich
 ``x += m · norm_b(sublayer(norm(x)))`` with token shift in front of the mixer.  The residual stream ``x`` is
 fp32; GEMM operands are the model dtype.  Tensor parallelism is not implemented for these stacks.
 """
@@ -165,7 +175,120 @@ class LightningAttention(nn.Module):
         return ops.linear(y, self.o.data)
 
 
-MIXERS = {"attention": WindowAttention, "latent_attention": LatentAttention, "lightning": LightningAttention}
+class SinkTalkAttention(nn.Module):
+    """``extra`` output columns are appended to the fused input projection (the layer's residual gate reads the same
+    input): ``forward`` returns ``(attention output [T, H·Dv] before the output projection's caller-side scaling, extra)``."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, ctx: ParallelContext, dtype, device, extra: int = 0):
+        super().__init__()
+        self.s, self.eps, self.extra = spec, eps, extra
+        H, G, D, Dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
+        assert H % G == 0, "query heads must be a multiple of the key/value heads"
+        assert spec.rot_dims % 2 == 0 and spec.rot_dims <= D
+        self.cols = (H * D, G * D, G * Dv, H * Dv, extra)           # q | k | v | output gate | extra
+        self.qkvg = _matrix(sum(self.cols), width, ctx, dtype, device)
+        self.o = _matrix(width, H * Dv, ctx, dtype, device)
+        self.q_norm, self.k_norm = _param((H * D,), ctx, device), _param((G * D,), ctx, device)
+        self.sink, self.talk = _param((H,), ctx, device), _param((H, H), ctx, device)
+        freq, self.mag = seqmix.stretched_inv_freq(spec.rot_base, spec.rot_dims, spec.rot_scaling, device)
+        self.register_buffer("inv_freq", freq, persistent=False)
+
+    def weights(self, p, extra_src=()):
+        yield p + "qkvg", self.qkvg, "normal", [p + "q", p + "k", p + "v", p + "g", *extra_src]
+        yield p + "o", self.o, "normal", None
+        yield p + "q.norm", self.q_norm, "ones", None
+        yield p + "k.norm", self.k_norm, "ones", None
+        yield p + "sink", self.sink, "zeros", None
+        yield p + "talk", self.talk, "eye", None
+
+    def cache(self, num_blocks, num_slots, dtype, device) -> LayerCache:
+        s = self.s
+        return LayerCache(k=torch.zeros(num_blocks, KV_BLOCK_SIZE, s.kv_heads * s.dim, dtype=dtype, device=device),
+                          v=torch.zeros(num_blocks, KV_BLOCK_SIZE, s.kv_heads * s.vdim, dtype=dtype, device=device))
+
+    def forward(self, h, meta, cache: LayerCache):
+        s = self.s
+        H, G, D, Dv = s.heads, s.kv_heads, s.dim, s.vdim
+        T = h.shape[0]
+        nq, nk, nv, ng, _ = self.cols
+        both = ops.linear(h, self.qkvg.data)
+        seqmix.wide_norm_rope_cache(both, self.q_norm.data, self.k_norm.data, self.eps, meta.positions, self.inv_freq, self.mag,
+                                    s.rot_dims, meta.slot_mapping, cache.k, cache.v, H, G, D, Dv)
+        out = torch.empty(T, H * Dv, dtype=h.dtype, device=h.device)
+        g0 = nq + nk + nv
+        seqmix.talk_attention(out, both[:, :nq].unflatten(1, (H, D)), both[:, g0:g0 + ng], cache.k, cache.v, meta, G, Dv, s.scale,
+                              self.sink.data, self.talk.data)
+        return ops.linear(out, self.o.data), both[:, g0 + ng:]
+
+
+class TimeMix(nn.Module):
+    BLENDS = "rkvgw"                                     # order of the blend rows: receptance, key, value, gate, decay
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, ctx: ParallelContext, dtype, device):
+        super().__init__()
+        self.s, self.eps = spec, eps
+        H, D = spec.heads, spec.dim
+        C = H * D
+        assert spec.lora > 0, "the decay projection needs a rank"
+        self.mu = _param((5, width), ctx, device)
+        self.rkvg = Weight((4, C, width), None, ctx, dtype, device)         # one batched product for the four wide projections
+        self.w1, self.w2 = _matrix(spec.lora, width, ctx, dtype, device), _matrix(C, spec.lora, ctx, dtype, device)
+        self.w0, self.u, self.norm = _param((C,), ctx, device), _param((C,), ctx, device), _param((C,), ctx, device)
+        self.o = _matrix(width, C, ctx, dtype, device)
+
+    def weights(self, p):
+        yield p + "mu", self.mu, "half", [[p + "mu." + s] for s in self.BLENDS]
+        yield p + "rkvg", self.rkvg, "normal", [[p + s] for s in "rkvg"]
+        yield p + "w1", self.w1, "normal", None
+        yield p + "w2", self.w2, "normal", None
+        yield p + "w0", self.w0, "zeros", None
+        yield p + "u", self.u, "half", None
+        yield p + "norm", self.norm, "ones", None
+        yield p + "o", self.o, "normal", None
+
+    def cache(self, num_blocks, num_slots, dtype, device) -> LayerCache:
+        s = self.s
+        return LayerCache(state=torch.zeros(num_slots, s.heads, s.dim, s.dim, dtype=torch.float32, device=device),
+                          shift=torch.zeros(num_slots, self.mu.data.shape[1], dtype=torch.float32, device=device))
+
+    def forward(self, h, meta, cache: LayerCache):
+        s = self.s
+        blends = seqmix.shift_mix(h, self.mu.data, cache.shift, meta)                    # [5, T, W]
+        rkvg = torch.bmm(blends[:4], self.rkvg.data.transpose(1, 2))                     # [4, T, C]
+        w = seqmix.decay_lora(ops.linear(blends[4], self.w1.data), self.w2.data, self.w0.data)
+        o = seqmix.wkv_scan(rkvg, w, self.u.data, cache.state, meta, s.heads, s.dim)
+        y = seqmix.group_rms_gate(o, s.heads, self.norm.data, self.eps, rkvg[3], h.dtype)
+        return ops.linear(y, self.o.data)
+
+
+class DualMixer(nn.Module):
+    """Sink attention and a time mix on the same input; ``forward`` returns both outputs (the layer's combine step applies
+    ``part_scales`` in fp32) and the extra columns of the attention's input projection."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, ctx: ParallelContext, dtype, device, extra: int = 0):
+        super().__init__()
+        kinds = tuple(p.kind for p in spec.parts)
+        if kinds != ("sink_attention", "time_mix"):
+            raise ValueError(f"parallel mixers are sink attention beside a time mix, not {kinds}")
+        self.s = spec
+        self.left = SinkTalkAttention(spec.parts[0], width, eps, ctx, dtype, device, extra)
+        self.right = TimeMix(spec.parts[1], width, eps, ctx, dtype, device)
+
+    def weights(self, p, extra_src=()):
+        yield from self.left.weights(p + "left.", extra_src)
+        yield from self.right.weights(p + "right.")
+
+    def cache(self, num_blocks, num_slots, dtype, device) -> LayerCache:
+        a, b = self.left.cache(num_blocks, num_slots, dtype, device), self.right.cache(num_blocks, num_slots, dtype, device)
+        return LayerCache(k=a.k, v=a.v, state=b.state, shift=b.shift)
+
+    def forward(self, h, meta, cache: LayerCache):
+        left, extra = self.left(h, meta, cache)
+        return [left, self.right(h, meta, cache)], extra
+
+
+MIXERS = {"attention": WindowAttention, "latent_attention": LatentAttention, "lightning": LightningAttention,
+          "sink_attention": SinkTalkAttention, "time_mix": TimeMix, "parallel": DualMixer}
 
 
 class DenseFF(nn.Module):
@@ -177,6 +300,84 @@ class DenseFF(nn.Module):
 
     def forward(self, h):
         return ops.linear(seqmix.relu2(ops.linear(h, self.up.data)), self.down.data)
+
+
+class RoutedFF(nn.Module):
+    """``Σ_chosen score · scale · expert(h)  +  sigmoid(w_sg · h) · shared(h)`` with ``expert(h) = W_down · relu(W_up h)²``;
+    scores are sigmoids of fp32 router logits, the ``top`` largest are chosen and not renormalised.  ``extra`` output
+    columns are appended to the shared expert's up projection (the layer's residual gate reads the same input)."""
+
+    def __init__(self, spec: MixerSpec, width: int, ctx, dtype, device, extra: int = 0):
+        super().__init__()
+        self.s, self.extra = spec, extra
+        E, F, Fs = spec.experts, spec.ff, spec.shared_ff
+        assert 1 <= spec.top <= E
+        self.up, self.down = Weight((E, F, width), None, ctx, dtype, device), Weight((E, width, F), None, ctx, dtype, device)
+        self.router = _param((E + (1 if Fs else 0), width), ctx, device)     # fp32; last row: the shared expert's gate
+        self.shared_up = _matrix(Fs + extra, width, ctx, dtype, device) if Fs + extra else None
+        self.shared_down = _matrix(width, Fs, ctx, dtype, device) if Fs else None
+
+    def weights(self, p, extra_src=()):
+        E, Fs = self.s.experts, self.s.shared_ff
+        yield p + "experts.up", self.up, "normal", [[p + f"e{e}.up"] for e in range(E)]
+        yield p + "experts.down", self.down, "normal", [[p + f"e{e}.down"] for e in range(E)]
+        yield p + "router", self.router, "normal", [p + "router"] + ([p + "shared.sg"] if Fs else [])
+        if self.shared_up is not None:
+            yield p + "shared.up", self.shared_up, "normal", ([p + "shared.up"] if Fs else []) + list(extra_src)
+        if Fs:
+            yield p + "shared.down", self.shared_down, "normal", None
+
+    def forward(self, h):
+        """Returns ``(routed sum [T, W], shared expert's output or None, its gate fp32 [T] or None, extra columns)``."""
+        s = self.s
+        ids, wts, sgate = seqmix.sigmoid_route(h, self.router.data, s.experts, s.top, s.router_scale)
+        routed = seqmix.relu2_experts(h, ids, wts, self.up.data, self.down.data)
+        shared = extra = None
+        if self.shared_up is not None:
+            both = ops.linear(h, self.shared_up.data)
+            extra = both[:, s.shared_ff:]
+            if s.shared_ff:
+                shared = ops.linear(seqmix.relu2_rows(both[:, :s.shared_ff]), self.shared_down.data)
+        return routed, shared, sgate, extra
+
+
+class GatedParallelLayer(nn.Module):
+    def __init__(self, spec: MixerSpec, width: int, eps: float, mult: float, ctx: ParallelContext, dtype, device):
+        super().__init__()
+        self.spec, self.eps, self.mult, self.dtype = spec, eps, mult, dtype
+        self.norm1, self.rg1_b = _param((1,), ctx, device), _param((width,), ctx, device)
+        self.mixer = DualMixer(spec, width, eps, ctx, dtype, device, extra=width)       # + the mixer's residual gate
+        self.ff = None
+        if spec.ff:
+            if spec.ff_kind != "moe":
+                raise ValueError(f"gated parallel layers take a routed feed-forward, not {spec.ff_kind!r}")
+            self.norm2, self.rg2_b = _param((1,), ctx, device), _param((width,), ctx, device)
+            self.ff = RoutedFF(spec, width, ctx, dtype, device, extra=width)             # + the feed-forward's residual gate
+
+    def weights(self, p):
+        yield p + "norm1", self.norm1, "ones", None
+        yield p + "rg1.b", self.rg1_b, "zeros", None
+        yield from self.mixer.weights(p + "mix.", extra_src=(p + "rg1",))
+        if self.ff is not None:
+            yield p + "norm2", self.norm2, "ones", None
+            yield p + "rg2.b", self.rg2_b, "zeros", None
+            yield from self.ff.weights(p + "mlp.", extra_src=(p + "rg2",))
+
+    def cache(self, num_blocks, num_slots, dtype, device) -> LayerCache:
+        return self.mixer.cache(num_blocks, num_slots, dtype, device)
+
+    def forward(self, x, restart, meta, cache: LayerCache):
+        """``x``: fp32 stream ``[T, W]``, updated in place."""
+        assert restart is None, "gated parallel layers are not repeated"
+        h1, h2 = seqmix.rms_scale(x, self.norm1.data, self.norm2.data if self.ff is not None else None, self.eps, self.dtype)
+        parts, gate1 = self.mixer(h1, meta, cache)
+        if self.ff is None:
+            seqmix.gated_combine(x, self.mult, parts, list(self.spec.part_scales), gate1, self.rg1_b.data)
+            return x
+        routed, shared, sgate, gate2 = self.ff(h2)
+        seqmix.gated_combine(x, self.mult, parts, list(self.spec.part_scales), gate1, self.rg1_b.data, routed, shared, sgate,
+                             gate2, self.rg2_b.data)
+        return x
 
 
 class MixerLayer(nn.Module):

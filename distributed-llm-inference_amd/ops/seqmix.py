@@ -276,3 +276,219 @@ def lightning_scan(qkvg: torch.Tensor, state: torch.Tensor, meta, H: int, D: int
             o[t] = torch.einsum("hde,hd->he", S, q[t])
         state[slots[i]] = S
     return o.view(T, H * Dv)
+
+
+# ====================================================================================== gated parallel layers
+# Ops of stacks whose layers run two mixers and a routed feed-forward side by side on scalar-gain RMS norms of the same
+# stream (``models/mixers.py``: ``SinkTalkAttention``, ``TimeMix``, ``RoutedFF``, ``GatedParallelLayer``).  GPU kernels:
+# ``csrc/kernels/dualmix.hip`` (``torch.ops.dli.dm_*``).
+def _seq_rows(meta):
+    """(batch row, first token row, end token row, state slot) of the step's sequences that bring tokens (CPU references)."""
+    B = meta.num_decode + meta.num_prefill
+    qsl = meta.query_start_loc[:B + 1].tolist()
+    slots = meta.state_slots[:B].tolist() if meta.state_slots is not None else [-1] * B
+    return [(i, qsl[i], qsl[i + 1], slots[i]) for i in range(B) if qsl[i + 1] > qsl[i]]
+
+
+def rms_scale(x: torch.Tensor, g1: torch.Tensor, g2: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype):
+    """Two scalar-gain RMS norms of the same fp32 rows: ``x / sqrt(mean(x²) + eps) · g`` for ``g1`` and (when given) ``g2``
+    (one-element fp32 tensors).  Returns ``(h1, h2 or None)`` in ``out_dtype``."""
+    if x.is_cuda:
+        h1, h2 = _hip().dm_rms_scale(x, g1, g2, eps, out_dtype == torch.bfloat16)
+        return h1, (h2 if g2 is not None else None)
+    n = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps)
+    return (n * g1).to(out_dtype), ((n * g2).to(out_dtype) if g2 is not None else None)
+
+
+def shift_mix(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, meta) -> torch.Tensor:
+    """``out[s, t] = h[t] + (h[t-1] - h[t]) · mu[s]`` for every blend ``s`` (``mu`` fp32 ``[S, W]``), ``h[t-1]`` being the
+    previous token of the same sequence: the row above inside a chunk, the sequence's fp32 ``state`` row at a chunk start,
+    zero at position 0.  The state row becomes ``h`` of the sequence's last token of this step.  Returns ``[S, T, W]``."""
+    if _act_ok(h):
+        return _hip().dm_shift_mix(h, mu, state, meta.positions, meta.token_seq, meta.query_start_loc, meta.state_slots,
+                                   meta.counts, meta.num_seqs)
+    hf = h.float()
+    prev = torch.zeros_like(hf)
+    prev[1:] = hf[:-1]
+    for _i, t0, t1, slot in _seq_rows(meta):
+        prev[t0] = state[slot] if int(meta.positions[t0]) > 0 else 0.0
+        state[slot] = hf[t1 - 1]
+    return (hf.unsqueeze(0) + (prev - hf).unsqueeze(0) * mu.unsqueeze(1)).to(h.dtype)
+
+
+def stretched_inv_freq(base: float, dims: int, scaling: tuple = (), device="cpu"):
+    """Rotation frequencies of ``dims`` rotated entries (float64 ``[dims/2]``) and the magnitude applied to cosine and sine.
+    ``scaling = (factor, original, fast, slow)``: pairs that turn more than ``fast`` times over ``original`` positions keep
+    their frequency, pairs that turn fewer than ``slow`` times have it divided by ``factor``, with a linear blend over the
+    pair index between the two corners; the magnitude is ``0.1 · ln(factor) + 1``."""
+    import math
+    f = rotary_inv_freq(base, dims, "cpu")
+    if not scaling:
+        return f.to(device), 1.0
+    factor, original, fast, slow = scaling
+
+    def corner(turns):
+        return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+
+    lo, hi = max(math.floor(corner(fast)), 0), min(math.ceil(corner(slow)), dims - 1)
+    ramp = ((torch.arange(dims // 2, dtype=torch.float64) - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    return (f / factor * ramp + f * (1.0 - ramp)).to(device), 0.1 * math.log(factor) + 1.0
+
+
+def wide_norm_rope_cache(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor, eps: float, positions: torch.Tensor,
+                         inv_freq: torch.Tensor, mag: float, rot_dims: int, slot_mapping: torch.Tensor, k_cache: torch.Tensor,
+                         v_cache: torch.Tensor, H: int, G: int, D: int, Dv: int) -> None:
+    """Leading columns of ``qkv`` rows = ``[q (H·D) | k (G·D) | v (G·Dv)]``.  The whole q row and the whole k row are each
+    divided by their root mean square (over all heads at once) and multiplied by ``qw`` / ``kw``; then entries ``i`` and
+    ``i + rot_dims/2`` (``i < rot_dims/2``) of every head are turned by ``position · inv_freq[i]`` with cosine and sine
+    scaled by ``mag``.  q is written back in place; k and v go to the token-major cache rows ``slot_mapping`` (< 0: skipped)."""
+    if _act_ok(qkv):
+        _hip().dm_wide_norm_rope_cache(qkv, qw, kw, eps, positions, inv_freq, mag, rot_dims, slot_mapping, k_cache, v_cache, H, G, D, Dv)
+        return
+    T = qkv.shape[0]
+    q, k = qkv[:, :H * D].float(), qkv[:, H * D:(H + G) * D].float()
+    q = (q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps) * qw).view(T, H, D)
+    k = (k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps) * kw).view(T, G, D)
+    if rot_dims:
+        ang = positions.double()[:, None] * inv_freq[None, :]
+        cos, sin = (ang.cos() * mag).float().unsqueeze(1), (ang.sin() * mag).float().unsqueeze(1)
+        half = rot_dims // 2
+
+        def turn(v):
+            a, b = v[..., :half], v[..., half:rot_dims]
+            return torch.cat([a * cos - b * sin, b * cos + a * sin, v[..., rot_dims:]], dim=-1)
+        q, k = turn(q), turn(k)
+    qkv[:, :H * D] = q.reshape(T, H * D).to(qkv.dtype)
+    keep = slot_mapping >= 0
+    s = slot_mapping[keep].long()
+    k_cache.view(-1, G * D)[s] = k.reshape(T, G * D)[keep].to(k_cache.dtype)
+    v_cache.view(-1, G * Dv)[s] = qkv[:, (H + G) * D:(H + G) * D + G * Dv][keep].to(v_cache.dtype)
+
+
+def talk_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: torch.Tensor,
+                   meta, G: int, Dv: int, scale: float, sink: Optional[torch.Tensor], talk: Optional[torch.Tensor]) -> torch.Tensor:
+    """Causal softmax attention of this step's tokens over their sequences' cached rows with a per-head ``sink`` in the
+    denominator (``p = exp(s) / (Σ exp(s) + exp(sink))``) and the normalised weights mixed across heads:
+    ``p'_h = Σ_g talk[h, g] · p_g``; head ``h`` applies ``p'_h`` to the values of its own key / value head ``h // (H/G)``.
+    ``q [T, H, D]`` (strided view); ``gate [T, H·Dv]`` (pre-activation): the result is multiplied by its sigmoid.
+    Writes ``out [T, H·Dv]``."""
+    if _act_ok(q):
+        _hip().dm_talk_attention(out, q, gate, k_cache, v_cache, meta.block_tables, meta.positions, meta.token_seq,
+                                 sink, talk, G, Dv, scale)
+        return out
+    T, H, D = q.shape
+    kflat, vflat = k_cache.view(-1, G * D), v_cache.view(-1, G * Dv)
+    rep = H // G
+    res = torch.zeros(T, H, Dv)
+    for i, t0, t1, _slot in _seq_rows(meta):
+        pos = meta.positions[t0:t1].long()
+        L = int(pos[-1]) + 1
+        j = torch.arange(L)
+        slots = meta.block_tables[i, j // KV_BLOCK_SIZE].long() * KV_BLOCK_SIZE + j % KV_BLOCK_SIZE
+        K = kflat[slots].float().view(L, G, D).repeat_interleave(rep, dim=1)
+        V = vflat[slots].float().view(L, G, Dv).repeat_interleave(rep, dim=1)
+        s = torch.einsum("nhd,lhd->nhl", q[t0:t1].float(), K) * scale
+        s = s.masked_fill((j[None, :] > pos[:, None]).unsqueeze(1), float("-inf"))
+        if sink is not None:
+            s = torch.cat([s, sink.view(1, H, 1).expand(t1 - t0, H, 1)], dim=-1)
+        p = torch.softmax(s, dim=-1)[..., :L]
+        if talk is not None:
+            p = torch.einsum("hg,ngl->nhl", talk, p)
+        res[t0:t1] = torch.einsum("nhl,lhd->nhd", p, V)
+    res = res.view(T, H * Dv)
+    if gate is not None:
+        res = res * torch.sigmoid(gate.float())
+    out.copy_(res.to(out.dtype))
+    return out
+
+
+def decay_lora(a: torch.Tensor, w2: torch.Tensor, w0: torch.Tensor) -> torch.Tensor:
+    """fp32 ``exp(-exp(w2 · tanh(a) + w0))``: ``a [T, L]`` is the low-rank projection's output, ``w2 [C, L]``, ``w0`` fp32 ``[C]``."""
+    if _act_ok(a):
+        return _hip().dm_decay(a, w2, w0)
+    return torch.exp(-torch.exp(torch.tanh(a.float()) @ w2.float().t() + w0))
+
+
+def wkv_scan(rkv: torch.Tensor, w: torch.Tensor, u: torch.Tensor, state: torch.Tensor, meta, H: int, D: int) -> torch.Tensor:
+    """``rkv [≥3, T, H·D]`` = receptance, key, value; ``w`` fp32 ``[T, H·D]`` decays; ``u`` fp32 ``[H·D]`` bonus.  Per sequence
+    and head, token by token, with ``S`` the sequence's fp32 ``state[slot, h]`` ``[D, D]`` (zero at position 0):
+    ``o[e] = Σ_d r[d] · (S[d, e] + u[d] k[d] v[e])``, then ``S[d, e] ← w[d] · S[d, e] + k[d] v[e]``.  Returns fp32 ``[T, H·D]``."""
+    if _act_ok(rkv):
+        return _hip().dm_wkv_scan(rkv, w, u, state, meta.positions, meta.query_start_loc, meta.state_slots, meta.counts,
+                                  meta.num_seqs, H, D)
+    T = rkv.shape[1]
+    r, k, v = (rkv[i].float().view(T, H, D) for i in range(3))
+    wv, uv = w.view(T, H, D), u.view(H, D)
+    o = torch.zeros(T, H, D)
+    for _i, t0, t1, slot in _seq_rows(meta):
+        S = state[slot].clone() if int(meta.positions[t0]) > 0 else torch.zeros(H, D, D)
+        for t in range(t0, t1):
+            kv = k[t].unsqueeze(2) * v[t].unsqueeze(1)
+            o[t] = torch.einsum("hde,hd->he", S + uv.unsqueeze(2) * kv, r[t])
+            S = wv[t].unsqueeze(2) * S + kv
+        state[slot] = S
+    return o.view(T, H * D)
+
+
+def group_rms_gate(o: torch.Tensor, groups: int, w: torch.Tensor, eps: float, gate: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """Every one of the ``groups`` equal slices of an fp32 row is divided by its own root mean square; the row is then
+    multiplied by ``w`` and by ``silu(gate)`` (``gate``: pre-activation rows, strided view)."""
+    if o.is_cuda:
+        return _hip().dm_group_rms_gate(o, groups, w, eps, gate, out_dtype == torch.bfloat16)
+    T, C = o.shape
+    g = o.view(T, groups, C // groups)
+    g = g * torch.rsqrt((g * g).mean(-1, keepdim=True) + eps)
+    return (g.reshape(T, C) * w * torch.nn.functional.silu(gate.float())).to(out_dtype)
+
+
+def sigmoid_route(h: torch.Tensor, router: torch.Tensor, experts: int, top: int, scale: float):
+    """fp32 ``s = sigmoid(router · h)`` per token; the ``top`` experts with the largest scores (ties: lowest index) and
+    their weights ``s · scale`` (not renormalised).  ``router`` fp32 ``[experts (+1), W]``: a last extra row is a per-token
+    gate, returned as its sigmoid.  Returns ``(ids int32 [T, top], weights fp32 [T, top], extra fp32 [T] or None)``."""
+    if _act_ok(h):
+        ids, wts, extra = _hip().dm_sigmoid_route(h, router, experts, top, scale)
+        return ids, wts, (extra if router.shape[0] > experts else None)
+    s = torch.sigmoid(h.float() @ router.t())
+    val, ids = torch.sort(s[:, :experts], dim=-1, descending=True, stable=True)
+    return ids[:, :top].int(), val[:, :top] * scale, (s[:, experts] if router.shape[0] > experts else None)
+
+
+def relu2_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, up: torch.Tensor, down: torch.Tensor) -> torch.Tensor:
+    """``Σ_slots wts[t, s] · down[e] · relu(up[e] · h[t])²`` with ``e = ids[t, s]``; ``up [E, F, W]``, ``down [E, W, F]``."""
+    if _act_ok(h):
+        return _hip().dm_relu2_experts(h, ids, wts, up, down)
+    out = torch.zeros(h.shape[0], h.shape[1])
+    hf = h.float()
+    for e in range(up.shape[0]):
+        tok, slot = torch.nonzero(ids == e, as_tuple=True)
+        if tok.numel():
+            a = torch.clamp(hf[tok] @ up[e].float().t(), min=0.0)
+            a = (a * a).to(h.dtype).float()
+            out.index_add_(0, tok, (a @ down[e].float().t()) * wts[tok, slot].unsqueeze(1))
+    return out.to(h.dtype)
+
+
+def relu2_rows(x: torch.Tensor) -> torch.Tensor:
+    """``max(x, 0)²`` of a row-strided 2-D view, as a contiguous tensor."""
+    if _act_ok(x):
+        return _hip().dm_relu2_rows(x)
+    z = torch.clamp(x.float(), min=0.0)
+    return (z * z).to(x.dtype)
+
+
+def gated_combine(x: torch.Tensor, mult: float, parts: list, scales: list, gate1: torch.Tensor, b1: torch.Tensor,
+                  ff: Optional[torch.Tensor] = None, shared: Optional[torch.Tensor] = None, shared_gate: Optional[torch.Tensor] = None,
+                  gate2: Optional[torch.Tensor] = None, b2: Optional[torch.Tensor] = None) -> None:
+    """In place on the fp32 stream: ``x += mult · (sigmoid(gate1 + b1) ⊙ Σ_i scales[i] · parts[i] + sigmoid(gate2 + b2) ⊙
+    (ff + shared_gate ⊙ shared))`` — the second term only with ``gate2``; ``shared_gate`` fp32 ``[T]`` (already a sigmoid)."""
+    if x.is_cuda:
+        assert len(parts) == 2, "the kernel combines two mixers"
+        _hip().dm_gated_combine(x, mult, parts[0], parts[1], scales[0], scales[1], gate1, b1, ff, shared, shared_gate, gate2, b2)
+        return
+    y = sum(s * p.float() for s, p in zip(scales, parts)) * torch.sigmoid(gate1.float() + b1)
+    if gate2 is not None:
+        f = ff.float() if ff is not None else 0.0
+        if shared is not None:
+            f = f + shared.float() * (shared_gate.unsqueeze(1) if shared_gate is not None else 1.0)
+        y = y + f * torch.sigmoid(gate2.float() + b2)
+    x.add_(y, alpha=mult)
