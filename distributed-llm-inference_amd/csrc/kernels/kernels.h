@@ -137,4 +137,36 @@ int launch_ep_dispatch(void* st, const void* x, int64_t x_stride, const int* ids
 int launch_ep_combine(void* st, const int* ids, const int* slot, int n, int n_cap, int H, int local_experts, void* y_back, int blocks,
                       hipStream_t stream);
 
+// gated parallel layers (dualmix.hip): same conventions as the seqmix launchers
+void launch_dm_rms_scale(const float* x, const float* g1, const float* g2, float eps, int rows, int W, void* h1, void* h2, bool out_bf16,
+                         hipStream_t stream);
+void launch_dm_shift_mix(const void* h, bool bf16, int64_t h_stride, const float* mu, int S, float* state, const int* positions,
+                         const int* token_seq, const int* qsl, const int* state_slots, const int* counts, int T, int seqs, int W,
+                         void* out, hipStream_t stream);
+void launch_dm_wide_norm_rope_cache(void* qkv, bool bf16, int64_t row_stride, const float* qw, const float* kw, float eps,
+                                    const int* positions, const double* freq, float mag, int rot_dims, const int* slot_mapping,
+                                    void* k_cache, void* v_cache, int rows, int H, int G, int D, int Dv, hipStream_t stream);
+size_t dm_talk_attention_lds(int H, int D);
+int dm_talk_attention_max_heads();
+int dm_talk_attention_max_out();
+void launch_dm_talk_attention(void* out, int64_t o_stride, const void* q, int64_t q_ts, int64_t q_hs, const void* gate, int64_t g_stride,
+                              const void* k_cache, const void* v_cache, bool bf16, const int* block_tables, int max_blocks,
+                              const int* positions, const int* token_seq, const float* sink, const float* talk, int rows, int H, int G,
+                              int D, int Dv, float scale, hipStream_t stream);
+void launch_dm_decay(const void* a, bool bf16, int64_t a_stride, const void* w2, const float* w0, int rows, int Lr, int C, float* out,
+                     hipStream_t stream);
+void launch_dm_wkv_scan(const void* rkv, bool bf16, int64_t plane, const float* w, const float* u, float* state, const int* positions,
+                        const int* qsl, const int* state_slots, const int* counts, int seqs, int H, int D, float* out,
+                        hipStream_t stream);
+void launch_dm_group_rms_gate(const float* o, int groups, const float* w, float eps, const void* gate, bool gate_bf16, int64_t g_stride,
+                              int rows, int C, void* out, bool out_bf16, hipStream_t stream);
+void launch_dm_sigmoid_route(const void* h, bool bf16, int64_t h_stride, const float* router, int router_rows, int E, int K, float scale,
+                             int rows, int W, int* ids, float* wts, float* extra, hipStream_t stream);
+void launch_dm_experts(const void* h, bool bf16, int64_t h_stride, const int* ids, const float* wts, int K, const void* up,
+                       const void* down, int rows, int F, int W, void* act, void* out, hipStream_t stream);
+void launch_dm_relu2_rows(const void* x, bool bf16, int64_t x_stride, int rows, int F, void* out, hipStream_t stream);
+void launch_dm_gated_combine(float* x, float mult, const void* p0, const void* p1, float s0, float s1, const void* g1, int64_t g1_stride,
+                             const float* b1, const void* ff, const void* shared, const float* sg, const void* g2, int64_t g2_stride,
+                             const float* b2, bool bf16, int rows, int W, hipStream_t stream);
+
 }  // namespace dli
