@@ -423,12 +423,12 @@ __global__ __launch_bounds__(NT) void sigmoid_route_kernel(const A* __restrict__
   __syncthreads();
   for (int r = wave; r < rows; r += NT / 64) {
     const float d = wave_dot<float>(sh, router + (int64_t)r * W, W);
-    if (lane == 0) z[r] = sigmoid_f(d);
+    if (lane == 0) z[r] = d;
   }
   __syncthreads();
   if (wave != 0) return;
-  if (rows > E && lane == 0) extra[t] = z[E];
-  float p = lane < E ? z[lane] : -1.f;
+  if (rows > E && lane == 0) extra[t] = sigmoid_f(z[E]);
+  float p = lane < E ? z[lane] : -3.0e38f;                  // picked by logit: the order of the scores, no saturated ties
   for (int k = 0; k < K; ++k) {
     float bv = p;
     int bi = lane;
@@ -440,9 +440,9 @@ __global__ __launch_bounds__(NT) void sigmoid_route_kernel(const A* __restrict__
     }
     if (lane == 0) {
       ids[t * K + k] = bi;
-      wts[t * K + k] = bv * scale;
+      wts[t * K + k] = sigmoid_f(bv) * scale;
     }
-    if (lane == bi) p = -2.f;
+    if (lane == bi) p = -3.2e38f;
   }
 }
 

@@ -448,9 +448,9 @@ def sigmoid_route(h: torch.Tensor, router: torch.Tensor, experts: int, top: int,
     if _act_ok(h):
         ids, wts, extra = _hip().dm_sigmoid_route(h, router, experts, top, scale)
         return ids, wts, (extra if router.shape[0] > experts else None)
-    s = torch.sigmoid(h.float() @ router.t())
-    val, ids = torch.sort(s[:, :experts], dim=-1, descending=True, stable=True)
-    return ids[:, :top].int(), val[:, :top] * scale, (s[:, experts] if router.shape[0] > experts else None)
+    z = h.float() @ router.t()
+    val, ids = torch.sort(z[:, :experts], dim=-1, descending=True, stable=True)   # by logit: the same order, no saturated ties
+    return ids[:, :top].int(), torch.sigmoid(val[:, :top]) * scale, (torch.sigmoid(z[:, experts]) if router.shape[0] > experts else None)
 
 
 def relu2_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, up: torch.Tensor, down: torch.Tensor) -> torch.Tensor:
