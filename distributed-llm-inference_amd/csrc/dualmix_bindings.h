@@ -78,10 +78,12 @@ void dm_wide_norm_rope_cache(Tensor qkv, const Tensor& qw, const Tensor& kw, dou
 
 void dm_talk_attention(Tensor out, const Tensor& q, const c10::optional<Tensor>& gate, const Tensor& k_cache, const Tensor& v_cache,
                        const Tensor& block_tables, const Tensor& positions, const Tensor& token_seq, const c10::optional<Tensor>& sink,
-                       const c10::optional<Tensor>& talk, int64_t G, int64_t Dv, double scale) {
+                       const c10::optional<Tensor>& talk, int64_t G, int64_t Dv, double scale, int64_t rows) {
   const bool bf = act_bf16(q, "q");
   TORCH_CHECK(q.dim() == 3 && q.stride(2) == 1, "q must be [T, H, D] with contiguous head rows");
   const int64_t T = q.size(0), H = q.size(1), D = q.size(2);
+  TORCH_CHECK(rows <= T, "more rows than tokens");
+  const int64_t todo = rows < 0 ? T : rows;                  // the leading rows this kernel serves (the tile kernel took the rest)
   TORCH_CHECK(G > 0 && H % G == 0 && Dv > 0, "heads must be a multiple of the key/value heads");
   check_act_like(out, bf, "out");
   check_rows(out, "out");
@@ -112,7 +114,56 @@ void dm_talk_attention(Tensor out, const Tensor& q, const c10::optional<Tensor>&
   TORCH_CHECK((int64_t)dli::dm_talk_attention_lds((int)H, (int)D) <= kSmMaxLds, "query rows too wide");
   dli::launch_dm_talk_attention(out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), q.stride(1), gp, gs, k_cache.data_ptr(),
                                 v_cache.data_ptr(), bf, block_tables.data_ptr<int>(), (int)block_tables.size(1), positions.data_ptr<int>(),
-                                token_seq.data_ptr<int>(), sp, tp, (int)T, (int)H, (int)G, (int)D, (int)Dv, (float)scale, cur_stream(q));
+                                token_seq.data_ptr<int>(), sp, tp, (int)todo, (int)H, (int)G, (int)D, (int)Dv, (float)scale, cur_stream(q));
+}
+
+// prefill tiles of a bf16 step on the matrix cores; false: not covered (nothing was launched)
+bool dm_talk_tile_attention(Tensor out, const Tensor& q, const c10::optional<Tensor>& gate, const Tensor& k_cache, const Tensor& v_cache,
+                            const Tensor& block_tables, const Tensor& seq_lens, const Tensor& qsl, const Tensor& tile_seq,
+                            const Tensor& tile_q0, int64_t num_tiles, const c10::optional<Tensor>& counts,
+                            const c10::optional<Tensor>& sink, const c10::optional<Tensor>& talk, int64_t G, int64_t Dv, double scale) {
+  if (!act_bf16(q, "q")) return false;
+  TORCH_CHECK(q.dim() == 3 && q.stride(2) == 1, "q must be [T, H, D] with contiguous head rows");
+  const int64_t T = q.size(0), H = q.size(1), D = q.size(2);
+  TORCH_CHECK(G > 0 && H % G == 0 && Dv > 0, "heads must be a multiple of the key/value heads");
+  check_act_like(out, true, "out");
+  check_rows(out, "out");
+  TORCH_CHECK(out.size(0) == T && out.size(1) == H * Dv, "out must be [T, H*Dv]");
+  const void* gp = nullptr;
+  int64_t gs = 0;
+  if (gate.has_value()) {
+    check_act_like(*gate, true, "gate");
+    check_rows(*gate, "gate");
+    TORCH_CHECK(gate->size(0) == T && gate->size(1) == H * Dv, "gate must be [T, H*Dv]");
+    gp = gate->data_ptr();
+    gs = gate->stride(0);
+  }
+  check_act_like(k_cache, true, "k_cache");
+  check_act_like(v_cache, true, "v_cache");
+  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() && k_cache.dim() == 3 && v_cache.dim() == 3 &&
+                  k_cache.size(1) == kSmPageTokens && v_cache.size(1) == kSmPageTokens && k_cache.size(2) == G * D &&
+                  v_cache.size(2) == G * Dv && k_cache.size(0) == v_cache.size(0),
+              "caches must be [pages, 32, G*D] and [pages, 32, G*Dv]");
+  check_i32(block_tables, "block_tables");
+  TORCH_CHECK(block_tables.dim() == 2, "block_tables must be [B, max_blocks]");
+  check_i32(seq_lens, "seq_lens");
+  check_i32(qsl, "query_start_loc");
+  check_i32(tile_seq, "tile_seq");
+  check_i32(tile_q0, "tile_q0");
+  TORCH_CHECK(num_tiles >= 0 && tile_seq.numel() >= num_tiles && tile_q0.numel() >= num_tiles, "tile list shorter than num_tiles");
+  TORCH_CHECK(qsl.numel() >= block_tables.size(0) + 1 && seq_lens.numel() >= block_tables.size(0), "batch-row metadata too short");
+  const int* cnt = nullptr;
+  if (counts.has_value()) {
+    check_i32(*counts, "counts");
+    TORCH_CHECK(counts->numel() >= 4, "counts too short");
+    cnt = counts->data_ptr<int>();
+  }
+  return dli::launch_dm_talk_tile_attention(out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), q.stride(1), gp, gs,
+                                            k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr<int>(),
+                                            (int)block_tables.size(1), seq_lens.data_ptr<int>(), qsl.data_ptr<int>(),
+                                            tile_seq.data_ptr<int>(), tile_q0.data_ptr<int>(), (int)num_tiles, cnt,
+                                            opt_f32(sink, "sink", H), opt_f32(talk, "talk", H * H), (int)H, (int)G, (int)D, (int)Dv,
+                                            (float)scale, cur_stream(q));
 }
 
 Tensor dm_decay(const Tensor& a, const Tensor& w2, const Tensor& w0) {
@@ -175,6 +226,9 @@ std::tuple<Tensor, Tensor, Tensor> dm_sigmoid_route(const Tensor& h, const Tenso
   return {ids, wts, extra};
 }
 
+bool g_dm_grouped_experts = true;     // A/B knob (dm_set_grouped_experts): routed experts as grouped GEMMs on the matrix cores
+void dm_set_grouped_experts(bool on) { g_dm_grouped_experts = on; }
+
 Tensor dm_relu2_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, const Tensor& up, const Tensor& down) {
   const bool bf = act_bf16(h, "h");
   check_rows(h, "h");
@@ -188,8 +242,37 @@ Tensor dm_relu2_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, c
   check_f32(wts, "wts");
   TORCH_CHECK(ids.dim() == 2 && ids.size(0) == T && wts.dim() == 2 && wts.size(0) == T && wts.size(1) == ids.size(1), "ids / wts must be [T, K]");
   const int64_t K = ids.size(1);
+  Tensor out = at::empty({T, W}, h.options());
+  if (bf && g_dm_grouped_experts && W % 128 == 0 && F % 128 == 0 && E <= 64 && T * K >= 64 && h.stride(0) % 8 == 0 &&
+      reinterpret_cast<uintptr_t>(h.data_ptr()) % 16 == 0) {
+    // matrix-core path: the routed rows are bucketed by expert and both projections run as grouped GEMMs on 128-row tiles
+    // (kernels/moe.hip: rows gathered by index, relu² in the first epilogue, gate weight and scatter in the second)
+    auto stream = cur_stream(h);
+    auto i32 = h.options().dtype(at::kInt);
+    const int64_t n = T * K, TR = 128;
+    const int64_t capacity = (n + TR - 1) / TR * TR + E * TR, max_tiles = capacity / TR;
+    Tensor sorted = at::empty({capacity}, i32), tile_expert = at::empty({max_tiles}, i32), meta = at::empty({2}, i32);
+    Tensor act = at::empty({capacity, F}, h.options());
+    const int64_t col_blocks2 = W / TR, nk2 = F / 64;
+    int64_t k_splits = 1;
+    if (max_tiles * col_blocks2 < 1024)
+      k_splits = std::min<int64_t>({(1024 + max_tiles * col_blocks2 - 1) / (max_tiles * col_blocks2), 16, nk2});
+    const bool split = k_splits > 1;
+    Tensor y = split ? at::empty({k_splits, n, W}, h.options().dtype(at::kFloat)) : at::empty({n, W}, h.options());
+    dli::launch_moe_align(ids.data_ptr<int>(), (int)n, 0, (int)E, sorted.data_ptr<int>(), tile_expert.data_ptr<int>(),
+                          meta.data_ptr<int>(), (int)capacity, (int)TR, stream);
+    dli::launch_grouped_gemm(3, h.data_ptr(), h.stride(0), up.data_ptr(), F * W, sorted.data_ptr<int>(), tile_expert.data_ptr<int>(),
+                             meta.data_ptr<int>(), wts.data_ptr<float>(), (int)K, act.data_ptr(), F, (int)W, (int)F, (int)max_tiles, 1, 0,
+                             stream);
+    dli::launch_grouped_gemm(split ? 2 : 1, act.data_ptr(), F, down.data_ptr(), W * F, sorted.data_ptr<int>(),
+                             tile_expert.data_ptr<int>(), meta.data_ptr<int>(), wts.data_ptr<float>(), (int)K, y.data_ptr(), W, (int)F,
+                             (int)W, (int)max_tiles, (int)k_splits, n * W, stream);
+    dli::launch_moe_sum(y.data_ptr(), split, (int)k_splits, n * W, ids.data_ptr<int>(), 0, (int)E, (int)K, (int)T, (int)W, out.data_ptr(),
+                        stream);
+    return out;
+  }
   TORCH_CHECK(W * 4 <= kSmMaxLds && K * F * 4 <= kSmMaxLds, "rows too wide");
-  Tensor act = at::empty({T * K, F}, h.options()), out = at::empty({T, W}, h.options());
+  Tensor act = at::empty({T * K, F}, h.options());
   dli::launch_dm_experts(h.data_ptr(), bf, h.stride(0), ids.data_ptr<int>(), wts.data_ptr<float>(), (int)K, up.data_ptr(), down.data_ptr(),
                          (int)T, (int)F, (int)W, act.data_ptr(), out.data_ptr(), cur_stream(h));
   return out;

@@ -302,6 +302,245 @@ __global__ __launch_bounds__(NT) void talk_attention_kernel(A* __restrict__ out,
   }
 }
 
+// ------------------------------------------------------------------------------------------------ attention: prefill tiles (bf16)
+// The same two passes on the matrix cores.  A workgroup owns 16 queries of one chunk and up to 16 output heads (grid.y:
+// groups of 16 heads); it computes the scores of ALL heads (the mixing needs them), a wave taking heads w, w+4, ….
+// Sᵀ = K·Qᵀ per head on v_mfma_f32_16x16x32_bf16 from a page of K rows staged in LDS (KG key heads per round); pass 1
+// keeps each head's running maximum and denominator per query; pass 2 writes the normalised fp32 weights of a page
+// to LDS [head][lane][8] — a lane's eight values (two 16-key tiles) are, in that order, its B fragment of the P·V k-step
+// — mixes them across heads in fp32 for the wave's own output heads, rounds the mixed weights to bf16 and accumulates
+// Oᵀ += Vᵀ·Pᵀ against the staged V page.  KS = D / 32, DVT = Dv / 16.
+constexpr int TT_MAX_HW = 8;        // score heads per wave → H ≤ 32
+constexpr int TT_HEADS = 16;        // output heads per workgroup
+constexpr int TT_MAX_HO = 4;        // output heads per wave
+
+template <int KS, int DVT>
+__global__ __launch_bounds__(NT) void talk_tile_kernel(
+    uint16_t* __restrict__ out, int64_t o_stride, const uint16_t* __restrict__ q, int64_t q_ts, int64_t q_hs,
+    const uint16_t* __restrict__ gate, int64_t g_stride, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
+    const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ seq_lens, const int* __restrict__ qsl,
+    const int* __restrict__ tile_seq, const int* __restrict__ tile_q0, int num_tiles, const int* __restrict__ counts,
+    const float* __restrict__ sink, const float* __restrict__ talk, int H, int G, int KG, int NVmax, float scale) {
+  extern __shared__ __align__(16) uint16_t tl[];
+  constexpr int D = 32 * KS, Dv = 16 * DVT;
+  const int ntiles = counts != nullptr ? min(counts[2], num_tiles) : num_tiles;
+  const int tile = num_tiles - 1 - (int)(blockIdx.x >> 2);        // the host lists causal tiles so that the END is longest
+  if (tile >= ntiles) return;
+  const int seq = tile_seq[tile];
+  const int q0 = tile_q0[tile] + 16 * (int)(blockIdx.x & 3);
+  const int t_begin = qsl[seq];
+  const int n_chunk = qsl[seq + 1] - t_begin;
+  const int nq = min(16, n_chunk - q0);
+  if (nq <= 0) return;
+  const int p0 = seq_lens[seq] - n_chunk;                          // position of the chunk's first token
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63, g4 = lane >> 4, c = lane & 15;
+  const int rep = H / G;
+  const int hb = blockIdx.y * TT_HEADS, nh = min(TT_HEADS, H - hb);
+  const int per = (nh + 3) >> 2;                                   // output heads per wave
+  const int c_lo = hb / rep, NV = (hb + nh - 1) / rep - c_lo + 1;  // value heads this workgroup reads
+  const int KST = KG * D + 8, VST = NVmax * Dv + 8;                // LDS row strides (elements): +16 bytes against bank conflicts
+  uint16_t* Ks = tl;
+  uint16_t* Vs = Ks + 32 * KST;
+  float* Pl = reinterpret_cast<float*>(Vs + 32 * VST);             // [H][64][8]
+  float* Tk = Pl + H * 512;                                        // [nh][H]
+  float* St = Tk + TT_HEADS * H;                                   // [H][16][2]: maximum, 1 / denominator
+  for (int i = threadIdx.x; i < nh * H; i += NT) {
+    const int h = hb + i / H, g = i % H;
+    Tk[i] = talk != nullptr ? talk[h * H + g] : (h == g ? 1.f : 0.f);
+  }
+  const bool qvalid = c < nq;
+  const int64_t tq = t_begin + q0 + (qvalid ? c : 0);
+  const int pos_q = qvalid ? p0 + q0 + c : 0x7fffffff;             // rows past the chunk: nothing masked, nothing stored
+  const int n_kb = (p0 + q0 + nq - 1) / kBlockTokens + 1;
+  const int* bt = block_tables + (int64_t)seq * max_blocks;
+  const int rounds = (G + KG - 1) / KG;
+  const int64_t krow = (int64_t)G * D, vrow = (int64_t)G * Dv;
+
+  // scores of head g for the staged K page: two 16-key tiles, natural units, masked entries → -inf
+#define TT_SCORES(g_, kvl_, kb_, s0_, s1_)                                                                         \
+  {                                                                                                                \
+    f32x4 a0_ = {0.f, 0.f, 0.f, 0.f}, a1_ = {0.f, 0.f, 0.f, 0.f};                                                  \
+    _Pragma("unroll") for (int ks_ = 0; ks_ < KS; ++ks_) {                                                         \
+      const bf16x8 qf_ = *reinterpret_cast<const bf16x8*>(q + tq * q_ts + (g_) * q_hs + ks_ * 32 + 8 * g4);        \
+      const bf16x8 k0_ = *reinterpret_cast<const bf16x8*>(Ks + c * KST + (kvl_) * D + ks_ * 32 + 8 * g4);          \
+      const bf16x8 k1_ = *reinterpret_cast<const bf16x8*>(Ks + (16 + c) * KST + (kvl_) * D + ks_ * 32 + 8 * g4);   \
+      a0_ = mfma16(k0_, qf_, a0_);                                                                                 \
+      a1_ = mfma16(k1_, qf_, a1_);                                                                                 \
+    }                                                                                                              \
+    _Pragma("unroll") for (int r_ = 0; r_ < 4; ++r_) {                                                             \
+      const int j_ = (kb_) * kBlockTokens + 4 * g4 + r_;                                                           \
+      s0_[r_] = j_ <= pos_q ? a0_[r_] * scale : -INFINITY;                                                         \
+      s1_[r_] = j_ + 16 <= pos_q ? a1_[r_] * scale : -INFINITY;                                                    \
+    }                                                                                                              \
+  }
+#define TT_STAGE_K(page_, r_)                                                                                      \
+  {                                                                                                                \
+    const int kg_ = min(KG, G - (r_) * KG), cpr_ = kg_ * D / 8;                                                    \
+    for (int i_ = threadIdx.x; i_ < 32 * cpr_; i_ += NT) {                                                         \
+      const int row_ = i_ / cpr_, ch_ = i_ - row_ * cpr_;                                                          \
+      *reinterpret_cast<bf16x8*>(Ks + row_ * KST + ch_ * 8) =                                                      \
+          *reinterpret_cast<const bf16x8*>(kc + ((int64_t)(page_) * kBlockTokens + row_) * krow + (r_) * KG * D + ch_ * 8); \
+    }                                                                                                              \
+  }
+
+  // ---- pass 1: maximum and denominator of every head
+  float m[TT_MAX_HW], l[TT_MAX_HW];
+#pragma unroll
+  for (int i = 0; i < TT_MAX_HW; ++i) { m[i] = -3.0e38f; l[i] = 0.f; }
+  for (int kb = 0; kb < n_kb; ++kb) {
+    const int page = bt[kb];
+    for (int r = 0; r < rounds; ++r) {
+      __syncthreads();
+      TT_STAGE_K(page, r);
+      __syncthreads();
+      const int g_lo = r * KG * rep, g_hi = min(H, g_lo + KG * rep);
+#pragma unroll
+      for (int i = 0; i < TT_MAX_HW; ++i) {
+        const int g = 4 * i + wave;
+        if (g >= g_lo && g < g_hi) {                              // wave-uniform
+          f32x4 s0, s1;
+          TT_SCORES(g, g / rep - r * KG, kb, s0, s1);
+          float mx = m[i];
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) mx = fmaxf(mx, fmaxf(s0[rr], s1[rr]));
+          float add = 0.f;
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) add += __expf(s0[rr] - mx) + __expf(s1[rr] - mx);
+          l[i] = l[i] * __expf(m[i] - mx) + add;
+          m[i] = mx;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < TT_MAX_HW; ++i) {
+    const int g = 4 * i + wave;
+    if (g < H) {
+      float mx = fmaxf(m[i], __shfl_xor(m[i], 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float sk = sink != nullptr ? sink[g] : -3.0e38f;
+      mx = fmaxf(mx, sk);
+      float ls = l[i] * __expf(m[i] - mx);
+      ls += __shfl_xor(ls, 16, 64);
+      ls += __shfl_xor(ls, 32, 64);
+      if (sink != nullptr) ls += __expf(sk - mx);
+      if (g4 == 0) {
+        St[(g * 16 + c) * 2] = mx;
+        St[(g * 16 + c) * 2 + 1] = 1.f / ls;
+      }
+    }
+  }
+
+  // ---- pass 2
+  f32x4 acc[TT_MAX_HO][DVT];
+#pragma unroll
+  for (int i = 0; i < TT_MAX_HO; ++i)
+#pragma unroll
+    for (int d = 0; d < DVT; ++d) acc[i][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int kb = 0; kb < n_kb; ++kb) {
+    const int page = bt[kb];
+    for (int r = 0; r < rounds; ++r) {
+      __syncthreads();                                            // everyone is done with the previous K / V / weights (and St is written)
+      TT_STAGE_K(page, r);
+      if (r == 0) {
+        const int cpr = NV * Dv / 8;
+        for (int i = threadIdx.x; i < 32 * cpr; i += NT) {
+          const int row = i / cpr, ch = i - row * cpr;
+          *reinterpret_cast<bf16x8*>(Vs + row * VST + ch * 8) =
+              *reinterpret_cast<const bf16x8*>(vc + ((int64_t)page * kBlockTokens + row) * vrow + c_lo * Dv + ch * 8);
+        }
+      }
+      __syncthreads();
+      const int g_lo = r * KG * rep, g_hi = min(H, g_lo + KG * rep);
+#pragma unroll
+      for (int i = 0; i < TT_MAX_HW; ++i) {
+        const int g = 4 * i + wave;
+        if (g >= g_lo && g < g_hi) {
+          f32x4 s0, s1;
+          TT_SCORES(g, g / rep - r * KG, kb, s0, s1);
+          const float mx = St[(g * 16 + c) * 2], il = St[(g * 16 + c) * 2 + 1];
+          f32x4 pa, pb;
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) {
+            pa[rr] = __expf(s0[rr] - mx) * il;
+            pb[rr] = __expf(s1[rr] - mx) * il;
+          }
+          *reinterpret_cast<f32x4*>(Pl + (g * 64 + lane) * 8) = pa;
+          *reinterpret_cast<f32x4*>(Pl + (g * 64 + lane) * 8 + 4) = pb;
+        }
+      }
+    }
+    __syncthreads();                                              // the page's weights of all heads are in LDS
+    int cur_c = -1;
+    bf16x8 vf[DVT];
+#pragma unroll
+    for (int i = 0; i < TT_MAX_HO; ++i) {
+      const int hl = wave * per + i;                              // wave-uniform
+      if (i < per && hl < nh) {
+        const float* trow = Tk + hl * H;
+        f32x4 ma = {0.f, 0.f, 0.f, 0.f}, mb = {0.f, 0.f, 0.f, 0.f};
+        for (int g = 0; g < H; ++g) {
+          const float tw = trow[g];
+          const f32x4 pa = *reinterpret_cast<const f32x4*>(Pl + (g * 64 + lane) * 8);
+          const f32x4 pb = *reinterpret_cast<const f32x4*>(Pl + (g * 64 + lane) * 8 + 4);
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) {
+            ma[rr] += tw * pa[rr];
+            mb[rr] += tw * pb[rr];
+          }
+        }
+        bf16x8 pf;
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          pf[rr] = (short)f2bf(ma[rr]);
+          pf[4 + rr] = (short)f2bf(mb[rr]);
+        }
+        const int cl = (hb + hl) / rep - c_lo;
+        if (cl != cur_c) {
+          cur_c = cl;
+#pragma unroll
+          for (int d = 0; d < DVT; ++d) {
+            const uint16_t* vp = Vs + cl * Dv + d * 16 + c;
+            bf16x8 v;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              v[j] = (short)vp[(4 * g4 + j) * VST];
+              v[4 + j] = (short)vp[(16 + 4 * g4 + j) * VST];
+            }
+            vf[d] = v;
+          }
+        }
+#pragma unroll
+        for (int d = 0; d < DVT; ++d) acc[i][d] = mfma16(vf[d], pf, acc[i][d]);
+      }
+    }
+  }
+#undef TT_SCORES
+#undef TT_STAGE_K
+  if (!qvalid) return;
+#pragma unroll
+  for (int i = 0; i < TT_MAX_HO; ++i) {
+    const int hl = wave * per + i;
+    if (i < per && hl < nh) {
+#pragma unroll
+      for (int d = 0; d < DVT; ++d) {
+        const int col = (hb + hl) * Dv + d * 16 + 4 * g4;
+        f32x4 o = acc[i][d];
+        if (gate != nullptr) {
+          const bf16x4 gv = *reinterpret_cast<const bf16x4*>(gate + tq * g_stride + col);
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) o[rr] *= sigmoid_f(bf2f((uint16_t)gv[rr]));
+        }
+        bf16x4 ov;
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) ov[rr] = (short)f2bf(o[rr]);
+        *reinterpret_cast<bf16x4*>(out + tq * o_stride + col) = ov;
+      }
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ decay
 // w[t, c] = exp(-exp(Σ_l w2[c, l] · tanh(a[t, l]) + w0[c]))
 template <typename A>
@@ -566,6 +805,49 @@ void launch_dm_talk_attention(void* out, int64_t o_stride, const void* q, int64_
   DM_BF16(bf16, A, hipLaunchKernelGGL(talk_attention_kernel<A>, dim3(rows), dim3(NT), dm_talk_attention_lds(H, D), stream, (A*)out, o_stride,
                                       (const A*)q, q_ts, q_hs, (const A*)gate, g_stride, (const A*)k_cache, (const A*)v_cache,
                                       block_tables, max_blocks, positions, token_seq, sink, talk, H, G, D, Dv, scale));
+}
+
+// Prefill tiles of a bf16 step on the matrix cores; false: shapes the tile kernel does not cover (the caller runs the
+// per-token kernel on every row instead).
+bool launch_dm_talk_tile_attention(void* out, int64_t o_stride, const void* q, int64_t q_ts, int64_t q_hs, const void* gate,
+                                   int64_t g_stride, const void* k_cache, const void* v_cache, const int* block_tables, int max_blocks,
+                                   const int* seq_lens, const int* qsl, const int* tile_seq, const int* tile_q0, int num_tiles,
+                                   const int* counts, const float* sink, const float* talk, int H, int G, int D, int Dv, float scale,
+                                   hipStream_t stream) {
+  if (num_tiles <= 0) return true;
+  const bool shape = (D == 64 && Dv == 64) || (D == 128 && Dv == 128);
+  if (!shape || H > 4 * TT_MAX_HW || H % G != 0) return false;
+  auto al = [](const void* p, int a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; };
+  if (!al(q, 16) || q_ts % 8 || q_hs % 8 || !al(out, 8) || o_stride % 4 || (gate != nullptr && (!al(gate, 8) || g_stride % 4)) ||
+      !al(k_cache, 16) || !al(v_cache, 16))
+    return false;
+  const int rep = H / G;
+  // key heads staged per round: the whole row when it fits 32 KiB, else groups whose query heads are a multiple of the 4 waves
+  int KG = G;
+  while (32 * KG * D * 2 > 32 * 1024 && KG % 2 == 0 && (KG / 2 * rep) % 4 == 0) KG /= 2;
+  if (32 * KG * D * 2 > 40 * 1024) return false;
+  const int groups = (H + TT_HEADS - 1) / TT_HEADS;
+  const int NVmax = std::min(G, (TT_HEADS + rep - 1) / rep + 1);
+  const size_t lds = (size_t)32 * (KG * D + 8) * 2 + (size_t)32 * (NVmax * Dv + 8) * 2 +
+                     (size_t)(H * 512 + TT_HEADS * H + H * 32) * sizeof(float);
+  if (lds > 150 * 1024) return false;
+#define DM_TT(KSV, DVTV)                                                                                                       \
+  do {                                                                                                                         \
+    static bool big = false;                                                                                                   \
+    if (!big) {                                                                                                                \
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&talk_tile_kernel<KSV, DVTV>),                                   \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);                                       \
+      big = true;                                                                                                              \
+    }                                                                                                                          \
+    hipLaunchKernelGGL((talk_tile_kernel<KSV, DVTV>), dim3(num_tiles * 4, groups), dim3(NT), lds, stream, (uint16_t*)out, o_stride, \
+                       (const uint16_t*)q, q_ts, q_hs, (const uint16_t*)gate, g_stride, (const uint16_t*)k_cache,              \
+                       (const uint16_t*)v_cache, block_tables, max_blocks, seq_lens, qsl, tile_seq, tile_q0, num_tiles, counts, \
+                       sink, talk, H, G, KG, NVmax, scale);                                                                    \
+  } while (0)
+  if (D == 64) DM_TT(2, 4);
+  else DM_TT(4, 8);
+#undef DM_TT
+  return true;
 }
 
 void launch_dm_decay(const void* a, bool bf16, int64_t a_stride, const void* w2, const float* w0, int rows, int Lr, int C, float* out,

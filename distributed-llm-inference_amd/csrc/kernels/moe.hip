@@ -133,7 +133,8 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
 }
 
 // ------------------------------------------------------------------------------------------ grouped GEMM
-enum { EPI_SWIGLU = 0, EPI_SCATTER = 1, EPI_SCATTER_SPLITK = 2 };   // SPLITK: fp32 partial slabs, summed by moe_sum
+enum { EPI_SWIGLU = 0, EPI_SCATTER = 1, EPI_SCATTER_SPLITK = 2, EPI_RELU2 = 3 };   // SPLITK: fp32 partial slabs, summed by moe_sum
+// EPI_RELU2: rows gathered like EPI_SWIGLU, 128 plain output columns per tile, stored as relu(·)² (experts without a gate)
 
 // byte offset of 16-byte chunk c (0..7) of row r inside a [128][64] bf16 LDS tile, XOR-swizzled so that
 // the 16 rows a ds_read_b128 lane group touches fall on different bank groups
@@ -188,7 +189,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(
   for (int i = 0; i < 4; ++i) {
     const int q = tid + 256 * i, r = q >> 3, c = (q & 7) ^ (r & 7);
     int64_t arow;
-    if (EPI == EPI_SWIGLU) {
+    if (EPI == EPI_SWIGLU || EPI == EPI_RELU2) {
       const int sid = sorted_ids[tile * BM + r];
       arow = sid >= 0 ? sid / top_k : 0;                     // padding rows read token 0 (discarded later)
     } else {
@@ -268,6 +269,18 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(
           o[r] = (short)f2bf(gate * fast_rcp(1.f + fast_exp2(-1.4426950408889634f * gate)) * up);
         }
         *reinterpret_cast<bf16x4*>(dst + n * 16) = o;           // padding rows hold finite junk, never read back
+      }
+    } else if (EPI == EPI_RELU2) {
+      uint16_t* dst = out + (int64_t)prow * out_stride + n0 + wn * 64 + 4 * g;
+#pragma unroll
+      for (int n = 0; n < 4; ++n) {
+        bf16x4 o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float a = fmaxf(acc[m][n][r], 0.f);
+          o[r] = (short)f2bf(a * a);
+        }
+        *reinterpret_cast<bf16x4*>(dst + n * 16) = o;
       }
     } else if (EPI == EPI_SCATTER_SPLITK) {
       if (sid >= 0) {
@@ -355,6 +368,7 @@ void launch_grouped_gemm(int epilogue, const void* A, int64_t a_stride, const vo
                      w_expert_stride, sorted_ids, tile_expert, meta, topk_w, top_k, out, out_stride, K, N_out, n_col_blocks, \
                      k_splits, slab_elems)
   if (epilogue == EPI_SWIGLU) DLI_GG(EPI_SWIGLU);
+  else if (epilogue == EPI_RELU2) DLI_GG(EPI_RELU2);
   else if (epilogue == EPI_SCATTER) DLI_GG(EPI_SCATTER);
   else DLI_GG(EPI_SCATTER_SPLITK);
 #undef DLI_GG

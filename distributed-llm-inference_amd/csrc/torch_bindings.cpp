@@ -609,7 +609,10 @@ TORCH_LIBRARY(dli, m) {
   m.def("dm_wide_norm_rope_cache(Tensor(a!) qkv, Tensor qw, Tensor kw, float eps, Tensor positions, Tensor freq, float mag, int rot_dims, "
         "Tensor slot_mapping, Tensor(b!) k_cache, Tensor(c!) v_cache, int H, int G, int D, int Dv) -> ()", &dm_wide_norm_rope_cache);
   m.def("dm_talk_attention(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor positions, "
-        "Tensor token_seq, Tensor? sink, Tensor? talk, int G, int Dv, float scale) -> ()", &dm_talk_attention);
+        "Tensor token_seq, Tensor? sink, Tensor? talk, int G, int Dv, float scale, int rows=-1) -> ()", &dm_talk_attention);
+  m.def("dm_talk_tile_attention(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor v_cache, Tensor block_tables, "
+        "Tensor seq_lens, Tensor qsl, Tensor tile_seq, Tensor tile_q0, int num_tiles, Tensor? counts, Tensor? sink, Tensor? talk, "
+        "int G, int Dv, float scale) -> bool", &dm_talk_tile_attention);
   m.def("dm_decay(Tensor a, Tensor w2, Tensor w0) -> Tensor", &dm_decay);
   m.def("dm_wkv_scan(Tensor rkv, Tensor w, Tensor u, Tensor(a!) state, Tensor positions, Tensor qsl, Tensor state_slots, Tensor counts, "
         "int num_seqs, int H, int D) -> Tensor", &dm_wkv_scan);
@@ -617,6 +620,7 @@ TORCH_LIBRARY(dli, m) {
   m.def("dm_sigmoid_route(Tensor h, Tensor router, int E, int K, float scale) -> (Tensor, Tensor, Tensor)", &dm_sigmoid_route);
   m.def("dm_relu2_experts(Tensor h, Tensor ids, Tensor wts, Tensor up, Tensor down) -> Tensor", &dm_relu2_experts);
   m.def("dm_relu2_rows(Tensor x) -> Tensor", &dm_relu2_rows);
+  m.def("dm_set_grouped_experts(bool on) -> ()", &dm_set_grouped_experts);
   m.def("dm_gated_combine(Tensor(a!) x, float mult, Tensor p0, Tensor p1, float s0, float s1, Tensor g1, Tensor b1, Tensor? ff, "
         "Tensor? shared, Tensor? sg, Tensor? g2, Tensor? b2) -> ()", &dm_gated_combine);
   m.def("fused_moe(Tensor x, Tensor router_logits, Tensor w13, Tensor w2, int top_k, int expert_offset, int tile_rows=0, Tensor? out=None) -> Tensor",

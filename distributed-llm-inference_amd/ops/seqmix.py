@@ -373,8 +373,17 @@ def talk_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Tens
     ``q [T, H, D]`` (strided view); ``gate [T, H·Dv]`` (pre-activation): the result is multiplied by its sigmoid.
     Writes ``out [T, H·Dv]``."""
     if _act_ok(q):
-        _hip().dm_talk_attention(out, q, gate, k_cache, v_cache, meta.block_tables, meta.positions, meta.token_seq,
-                                 sink, talk, G, Dv, scale)
+        lib = _hip()
+        rows = -1
+        if TILE_ATTENTION and q.dtype == torch.bfloat16 and meta.num_prefill_tiles > 0:
+            # prefill chunks: 16-query tiles on the matrix cores; the per-token kernel keeps the decode rows in front
+            if lib.dm_talk_tile_attention(out, q, gate, k_cache, v_cache, meta.block_tables, meta.seq_lens, meta.query_start_loc,
+                                          meta.prefill_tile_seq, meta.prefill_tile_q0, meta.num_prefill_tiles,
+                                          meta.counts if meta.counts_on_device else None, sink, talk, G, Dv, scale):
+                rows = meta.num_decode
+        if rows != 0:
+            lib.dm_talk_attention(out, q, gate, k_cache, v_cache, meta.block_tables, meta.positions, meta.token_seq,
+                                  sink, talk, G, Dv, scale, rows)
         return out
     T, H, D = q.shape
     kflat, vflat = k_cache.view(-1, G * D), v_cache.view(-1, G * Dv)
