@@ -9,6 +9,7 @@
         bench.py --gpus 8 --steps K --warmup W        # the driver's launch: ranks already exist
     python bench.py --sweep                           # SLO frontier: largest offered QPS with ≥ 90 % attainment
     python bench.py --mixers [--sizes small ...]      # side benchmark: Rodelix stacks beside Llama at equal layer sizes
+    python bench.py --mixers --models mixtral,vibunex # side benchmark: Vibunex stacks beside Mixtral at equal layer sizes
 
 One rank per GPU.  ``--tp`` consecutive ranks form one tensor-parallel replica (``dp = gpus / tp`` replicas);
 every replica serves its share (round-robin, the router's stateless policy) of ONE global BurstGPT-like trace

@@ -195,7 +195,10 @@ __global__ __launch_bounds__(NT) void talk_attention_kernel(A* __restrict__ out,
   extern __shared__ float sh[];
   const int t = blockIdx.x;
   const int seq = token_seq[t];
-  if (seq < 0) return;
+  if (seq < 0) {                                               // padding row of a captured step: zeros, not what the buffer held
+    for (int o = threadIdx.x; o < H * Dv; o += NT) stf<A>(out + (int64_t)t * o_stride + o, 0.f);
+    return;
+  }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int L = positions[t] + 1;
   const int rep = H / G;
@@ -667,21 +670,30 @@ __global__ __launch_bounds__(NT) void sigmoid_route_kernel(const A* __restrict__
   __syncthreads();
   if (wave != 0) return;
   if (rows > E && lane == 0) extra[t] = sigmoid_f(z[E]);
-  float p = lane < E ? z[lane] : -3.0e38f;                  // picked by logit: the order of the scores, no saturated ties
+  // Picked by logit (the order of the scores, no saturated ties).  Every round takes an expert that is still free, whatever
+  // the logits hold: a row of padding can carry NaNs, and an id outside the experts would index past their weights.  A lane
+  // that cannot be picked (no expert, or taken) offers -inf under an index past every expert; a NaN logit counts as -inf.
+  float p = -INFINITY;
+  if (lane < E) {
+    const float v = z[lane];
+    p = v == v ? v : -INFINITY;
+  }
+  bool free_lane = lane < E;
   for (int k = 0; k < K; ++k) {
-    float bv = p;
-    int bi = lane;
+    float bv = free_lane ? p : -INFINITY;
+    int bi = free_lane ? lane : 64 + lane;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
       const float ov = __shfl_xor(bv, o, 64);
       const int oi = __shfl_xor(bi, o, 64);
       if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
     }
+    // (value, index) is a total order without NaNs: every lane now holds the same pick
     if (lane == 0) {
-      ids[t * K + k] = bi;
+      ids[t * K + k] = min(bi, E - 1);
       wts[t * K + k] = sigmoid_f(bv) * scale;
     }
-    if (lane == bi) p = -3.2e38f;
+    if (lane == bi) free_lane = false;
   }
 }
 

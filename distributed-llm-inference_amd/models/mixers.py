@@ -214,7 +214,7 @@ class SinkTalkAttention(nn.Module):
         both = ops.linear(h, self.qkvg.data)
         seqmix.wide_norm_rope_cache(both, self.q_norm.data, self.k_norm.data, self.eps, meta.positions, self.inv_freq, self.mag,
                                     s.rot_dims, meta.slot_mapping, cache.k, cache.v, H, G, D, Dv)
-        out = torch.empty(T, H * Dv, dtype=h.dtype, device=h.device)
+        out = torch.zeros(T, H * Dv, dtype=h.dtype, device=h.device)     # padding rows of a captured step stay zero
         g0 = nq + nk + nv
         seqmix.talk_attention(out, both[:, :nq].unflatten(1, (H, D)), both[:, g0:g0 + ng], cache.k, cache.v, meta, G, Dv, s.scale,
                               self.sink.data, self.talk.data)

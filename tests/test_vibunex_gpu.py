@@ -110,3 +110,54 @@ def test_grouped_experts_against_the_row_kernels():
         err = ((got - want).norm() / want.norm()).item()
         assert err < 1e-2, f"{name}: {err}"
     assert not torch.equal(grouped, rows), "both calls took the same kernels"
+
+
+class _NamedOps:
+    """The kernel library with every call announced (flushed) and finished before the next: a fault then names its op."""
+
+    def __init__(self, lib):
+        self._lib = lib
+
+    def __getattr__(self, name):
+        fn = getattr(self._lib, name)
+        if not callable(fn):
+            return fn
+
+        def call(*a, **k):
+            print(f"    op {name}", flush=True)
+            out = fn(*a, **k)
+            torch.cuda.synchronize()
+            return out
+        return call
+
+
+@pytest.mark.skip(reason="a benchmark run of a stack with these layer sizes ended in an illegal memory access after the start-up "
+                         "checks had passed; the kernel was not identified, so nothing of that size runs on a GPU until it is")
+def test_layer_sizes_of_a_real_model_against_the_cpu_path(tmp_path, monkeypatch):
+    """One layer at the sizes of a real model (width 2048, 16 query / 4 key heads of 128, 32 recurrent heads of 64, 8 experts
+    of 5632, shared 1024): a 2 × 1100-token prefill step, decode steps of 2 rows and a mixed step, kernels against the CPU
+    path of the same ops (which the other tests pin to the oracle)."""
+    import numpy as np
+    from dli_amd.ops import seqmix
+    from rodelix_common import Rig, tokens
+    layer = {"type": "parallel",
+             "mixer": {"left_scale": 0.7, "right_scale": 0.7,
+                       "left": {"heads": 16, "kv_heads": 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                                "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}},
+                       "right": {"heads": 32, "dim": 64, "lora": 64}},
+             "mlp": {"kind": "moe", "expert": {"ff": 5632}, "router": {"experts": 8, "top": 2, "scale": 1.0}, "shared": {"ff": 1024}}}
+    cfg = cases.make_cfg([layer], width=2048, vocab=512, mult=0.5)
+    print("  writing the checkpoint", flush=True)
+    cases.write_checkpoint(tmp_path, cfg, seed=31, bf16=True)
+    reqs = {"a": tokens(1104, 512, 1), "b": tokens(1103, 512, 2), "c": tokens(70, 512, 3)}
+    sched = [[("a", 1100), ("b", 1100)], [("a", 1), ("b", 1)], [("a", 1), ("b", 1), ("c", 70)], [("a", 1), ("b", 1)], [("a", 1)]]
+    print("  cpu path", flush=True)
+    want = Rig(tmp_path, "bfloat16", "cpu", max_tokens=2560).run(reqs, sched)
+    print("  gpu path", flush=True)
+    rig = Rig(tmp_path, "bfloat16", "cuda", max_tokens=2560)
+    lib = seqmix._hip()
+    monkeypatch.setattr(seqmix, "_hip", lambda: _NamedOps(lib))
+    got = rig.run(reqs, sched)
+    for i in reqs:
+        e = cases._row_err(got[i], want[i])
+        assert np.median(e) < 2e-2 and (e > 6e-2).mean() < 0.1, f"{i}: median {np.median(e):.3e}, worst {e.max():.3e}"
