@@ -117,6 +117,8 @@ void dm_talk_attention(Tensor out, const Tensor& q, const c10::optional<Tensor>&
                                 token_seq.data_ptr<int>(), sp, tp, (int)todo, (int)H, (int)G, (int)D, (int)Dv, (float)scale, cur_stream(q));
 }
 
+void dm_prepare() { dli::dm_prepare_kernels(); }
+
 // prefill tiles of a bf16 step on the matrix cores; false: not covered (nothing was launched)
 bool dm_talk_tile_attention(Tensor out, const Tensor& q, const c10::optional<Tensor>& gate, const Tensor& k_cache, const Tensor& v_cache,
                             const Tensor& block_tables, const Tensor& seq_lens, const Tensor& qsl, const Tensor& tile_seq,

@@ -819,6 +819,19 @@ void launch_dm_talk_attention(void* out, int64_t o_stride, const void* q, int64_
                                       block_tables, max_blocks, positions, token_seq, sink, talk, H, G, D, Dv, scale));
 }
 
+// More than 64 KiB of dynamic LDS needs an opt-in per kernel.  Done once, for every instantiation, and callable ahead of time
+// (model construction) so that the attribute call never falls inside a stream capture.
+void dm_prepare_kernels() {
+  static const bool done = [] {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&talk_tile_kernel<2, 4>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              150 * 1024);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&talk_tile_kernel<4, 8>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              150 * 1024);
+    return true;
+  }();
+  (void)done;
+}
+
 // Prefill tiles of a bf16 step on the matrix cores; false: shapes the tile kernel does not cover (the caller runs the
 // per-token kernel on every row instead).
 bool launch_dm_talk_tile_attention(void* out, int64_t o_stride, const void* q, int64_t q_ts, int64_t q_hs, const void* gate,
@@ -843,14 +856,9 @@ bool launch_dm_talk_tile_attention(void* out, int64_t o_stride, const void* q, i
   const size_t lds = (size_t)32 * (KG * D + 8) * 2 + (size_t)32 * (NVmax * Dv + 8) * 2 +
                      (size_t)(H * 512 + TT_HEADS * H + H * 32) * sizeof(float);
   if (lds > 150 * 1024) return false;
+  dm_prepare_kernels();
 #define DM_TT(KSV, DVTV)                                                                                                       \
   do {                                                                                                                         \
-    static bool big = false;                                                                                                   \
-    if (!big) {                                                                                                                \
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&talk_tile_kernel<KSV, DVTV>),                                   \
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);                                       \
-      big = true;                                                                                                              \
-    }                                                                                                                          \
     hipLaunchKernelGGL((talk_tile_kernel<KSV, DVTV>), dim3(num_tiles * 4, groups), dim3(NT), lds, stream, (uint16_t*)out, o_stride, \
                        (const uint16_t*)q, q_ts, q_hs, (const uint16_t*)gate, g_stride, (const uint16_t*)k_cache,              \
                        (const uint16_t*)v_cache, block_tables, max_blocks, seq_lens, qsl, tile_seq, tile_q0, num_tiles, counts, \

@@ -153,6 +153,7 @@ void launch_dm_talk_attention(void* out, int64_t o_stride, const void* q, int64_
                               const void* k_cache, const void* v_cache, bool bf16, const int* block_tables, int max_blocks,
                               const int* positions, const int* token_seq, const float* sink, const float* talk, int rows, int H, int G,
                               int D, int Dv, float scale, hipStream_t stream);
+void dm_prepare_kernels();
 bool launch_dm_talk_tile_attention(void* out, int64_t o_stride, const void* q, int64_t q_ts, int64_t q_hs, const void* gate,
                                    int64_t g_stride, const void* k_cache, const void* v_cache, const int* block_tables, int max_blocks,
                                    const int* seq_lens, const int* qsl, const int* tile_seq, const int* tile_q0, int num_tiles,

@@ -613,6 +613,7 @@ TORCH_LIBRARY(dli, m) {
   m.def("dm_talk_tile_attention(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor v_cache, Tensor block_tables, "
         "Tensor seq_lens, Tensor qsl, Tensor tile_seq, Tensor tile_q0, int num_tiles, Tensor? counts, Tensor? sink, Tensor? talk, "
         "int G, int Dv, float scale) -> bool", &dm_talk_tile_attention);
+  m.def("dm_prepare() -> ()", &dm_prepare);
   m.def("dm_decay(Tensor a, Tensor w2, Tensor w0) -> Tensor", &dm_decay);
   m.def("dm_wkv_scan(Tensor rkv, Tensor w, Tensor u, Tensor(a!) state, Tensor positions, Tensor qsl, Tensor state_slots, Tensor counts, "
         "int num_seqs, int H, int D) -> Tensor", &dm_wkv_scan);

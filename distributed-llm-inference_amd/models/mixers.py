@@ -192,6 +192,8 @@ class SinkTalkAttention(nn.Module):
         self.sink, self.talk = _param((H,), ctx, device), _param((H, H), ctx, device)
         freq, self.mag = seqmix.stretched_inv_freq(spec.rot_base, spec.rot_dims, spec.rot_scaling, device)
         self.register_buffer("inv_freq", freq, persistent=False)
+        if torch.device(device).type == "cuda":
+            seqmix._hip().dm_prepare()                      # kernel attributes are set outside any later stream capture
 
     def weights(self, p, extra_src=()):
         yield p + "qkvg", self.qkvg, "normal", [p + "q", p + "k", p + "v", p + "g", *extra_src]
