@@ -23,6 +23,10 @@ def test_unequal_requests_in_one_batch(tmp_path):
     cases.case_mixed_batch(tmp_path, "cpu", "float32")
 
 
+def test_chunks_beside_single_tokens_with_heads_of_64(tmp_path):
+    cases.case_mixed_batch_on_tiles(tmp_path, "cpu", "float32")
+
+
 def test_pages_and_slots_used_again(tmp_path):
     cases.case_reuse(tmp_path, "cpu", "float32")
 

@@ -33,6 +33,11 @@ def test_unequal_requests_in_one_batch(tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_chunks_beside_single_tokens_with_heads_of_64(tmp_path, dtype):
+    cases.case_mixed_batch_on_tiles(tmp_path, "cuda", dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_pages_and_slots_used_again(tmp_path, dtype):
     cases.case_reuse(tmp_path, "cuda", dtype)
 

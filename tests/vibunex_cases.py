@@ -129,6 +129,21 @@ def case_mixed_batch(tmp, device, dtype):
         _check(got[i], want[i], dtype, f"request {i} in mixed batches")
 
 
+def case_mixed_batch_on_tiles(tmp, device, dtype):
+    """Chunks of two sequences beside decode rows of others in one step, with heads of 64 (on the GPU in bf16: the chunks
+    take the matrix-core tile kernel, the single tokens the per-token kernel)."""
+    cfg = other_size_configs()["matrix-core tiles, heads of 64 in two groups, no feed-forward"]
+    W, rig = _setup(tmp, cfg, dtype, device, seed=21, max_tokens=640)
+    reqs = {"a": tokens(150, cfg["vocab"], 50), "b": tokens(97, cfg["vocab"], 51), "c": tokens(40, cfg["vocab"], 52),
+            "d": tokens(3, cfg["vocab"], 53)}
+    want = {i: expect(cfg, W, t) for i, t in reqs.items()}
+    sched = [[("a", 70), ("c", 33)], [("a", 1), ("b", 64), ("c", 1), ("d", 1)], [("a", 50), ("b", 1), ("c", 1), ("d", 2)],
+             [("a", 1), ("b", 32), ("c", 5)], [("a", 28)]]
+    got = rig.run(reqs, sched)
+    for i in reqs:
+        _check(got[i], want[i], dtype, f"request {i} beside the others", strict=True)
+
+
 # ---------------------------------------------------------------- pages and state slots freed and used again
 def case_reuse(tmp, device, dtype):
     W, rig = _setup(tmp, FULL, dtype, device, seed=9, max_tokens=160, max_seqs=2)      # five pages, two slots
