@@ -53,8 +53,8 @@ def vibunex_raw(width, heads, kv, ffn):
     layer = {"type": "parallel",
              "mixer": {"left_scale": 0.7, "right_scale": 0.7,
                        "left": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
-                                "rot": {"base": 500000.0, "dims": 64,
-                                        "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}},
+                                "rot": {"base": 1000000.0, "dims": 64,
+                                        "scaling": {"factor": 8.0, "original": 8192, "fast": 16.0, "slow": 2.0}}},
                        "right": {"heads": width // 64, "dim": 64, "lora": 64}},
              "mlp": {"kind": "moe", "expert": {"ff": inner * 3 // 2 - 512}, "router": {"experts": 8, "top": 2, "scale": 1.0},
                      "shared": {"ff": 1024}}}

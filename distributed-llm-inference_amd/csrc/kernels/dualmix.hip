@@ -670,7 +670,7 @@ __global__ __launch_bounds__(NT) void sigmoid_route_kernel(const A* __restrict__
   __syncthreads();
   if (wave != 0) return;
   if (rows > E && lane == 0) extra[t] = sigmoid_f(z[E]);
-  // Picked by logit (the order of the scores, no saturated ties).  Every round takes an expert that is still free, whatever
+  // Picked by logit (the order of the scores, no saturated ties).  Every pass takes an expert that is still free, whatever
   // the logits hold: a row of padding can carry NaNs, and an id outside the experts would index past their weights.  A lane
   // that cannot be picked (no expert, or taken) offers -inf under an index past every expert; a NaN logit counts as -inf.
   float p = -INFINITY;

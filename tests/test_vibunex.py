@@ -72,7 +72,7 @@ def test_config_reader(tmp_path):
 def test_stretched_frequencies_against_the_oracle():
     from dli_amd.ops import seqmix
     for rot in ({"base": 8000.0, "dims": 12, "scaling": {"factor": 3.0, "original": 48, "fast": 8.0, "slow": 2.0}},
-                {"base": 500.0, "dims": 32, "scaling": {"factor": 16.0, "original": 4096, "fast": 32.0, "slow": 1.0}},
+                {"base": 500.0, "dims": 32, "scaling": {"factor": 16.0, "original": 4096, "fast": 24.0, "slow": 1.5}},
                 {"base": 10000.0, "dims": 6}):
         want, mag = oracle.stretched_frequencies(rot)
         sc = rot.get("scaling")

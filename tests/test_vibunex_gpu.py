@@ -148,7 +148,7 @@ def test_layer_sizes_of_a_real_model_against_the_cpu_path(tmp_path, monkeypatch)
     layer = {"type": "parallel",
              "mixer": {"left_scale": 0.7, "right_scale": 0.7,
                        "left": {"heads": 16, "kv_heads": 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
-                                "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}},
+                                "rot": {"base": 1000000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 8192, "fast": 16.0, "slow": 2.0}}},
                        "right": {"heads": 32, "dim": 64, "lora": 64}},
              "mlp": {"kind": "moe", "expert": {"ff": 5632}, "router": {"experts": 8, "top": 2, "scale": 1.0}, "shared": {"ff": 1024}}}
     cfg = cases.make_cfg([layer], width=2048, vocab=512, mult=0.5)
